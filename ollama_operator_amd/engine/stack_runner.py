@@ -24,8 +24,8 @@ import time
 
 import torch
 
-from ..models.config import (BLOCK_POSTNORM, FF_DENSE, MIX_ATTENTION, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM,
-                             MIX_RETENTION)
+from ..models.config import (BLOCK_POSTNORM, BLOCK_SANDWICH, FF_DENSE, FF_GLU, MIX_ATTENTION, MIX_LATENT, MIX_MAMBA2,
+                             MIX_MLSTM, MIX_RETENTION)
 from .runner import Runner
 from .weights import StackWeights
 
@@ -45,11 +45,15 @@ class StackExec:
         p = lambda t: t.data_ptr() if t is not None else 0  # noqa: E731
         e.configure(dict(E=cfg.n_embd, V=cfg.n_vocab, eps=float(cfg.norm_eps), residual_mult=float(cfg.residual_mult),
                          logit_softcap=float(cfg.logit_softcap), f32=int(w.dtype == torch.float32),
-                         max_B=r.max_batch, max_seqs=r.max_seqs, block=int(cfg.block), embed_scale=float(cfg.embed_scale)))
+                         max_B=r.max_batch, max_seqs=r.max_seqs, block=int(cfg.block), embed_scale=float(cfg.embed_scale),
+                         logit_scale=float(cfg.logit_scale), canon_taps=int(cfg.canon_taps)))
         e.set_globals(dict(embed=p(w.embed), loop_in=p(w.loop_in), final_w=p(w.final_w), final_b=p(w.final_b),
                            head=p(w.head)))
         for i, (L, spec) in enumerate(zip(w.layers, cfg.layers)):
             m, f = spec.mixer, spec.mlp
+            if cfg.block == BLOCK_SANDWICH:
+                e.set_layer(i, self._sandwich_layer(L, spec, p))
+                continue
             d = dict(kind=m.kind, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale,
                      softcap=m.softcap, qtemp_coef=m.qtemp_coef, qtemp_every=m.qtemp_every, rot_dims=m.rot_dims,
                      n_in=L["n_in"], norm_w=p(L["norm_w"]), norm_b=p(L["norm_b"]), w_in=p(L["w_in"]), w_o=p(L["w_o"]),
@@ -85,6 +89,7 @@ class StackExec:
                              ret_sin=p(r.ret_sin), ret_u_stride=r.ret_u.shape[1], cbuf=p(r.cbuf), ld_cbuf=r.cbuf.shape[1],
                              lat=p(r.latbuf), ld_lat=r.latbuf.shape[1], idw=p(r.idw), coef=p(r.scan_coef),
                              ld_coef=(r.scan_coef.shape[1] if r.scan_coef is not None else 0), ctot=p(r.scan_ctot),
+                             hn=p(r.hn), y2=p(r.ybuf2),
                              **{"moe_" + k: (v if isinstance(v, int) else p(v)) for k, v in r.moe_ws.items()}))
         e.set_inputs(dict(tokens=p(r.d_tokens), pos=p(r.d_pos), slot=p(r.d_slot), q_len=p(r.d_qlen),
                           q_seq=p(r.d_qseq), block_table=p(r.d_block_table), max_blocks=r.max_blocks,
@@ -94,6 +99,28 @@ class StackExec:
         self.chunk_rows = C.retention_chunk_rows()
         self.tile_rows = C.FLASH_TILE_ROWS
         e.bind_tiles(p(r.d_tiles), r.d_tiles.shape[0])
+
+    @staticmethod
+    def _sandwich_layer(L: dict, spec, p) -> dict:
+        """Descriptor of a layer with scalar-weight norms around both sublayers (csrc/stack LayerDesc)."""
+        m, f = spec.mixer, spec.mlp
+        d = dict(kind=m.kind, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale, rot_dims=m.rot_dims,
+                 n_in=L["n_in"], w_in=p(L["w_in"]), w_o=p(L["w_o"]), in_b=p(L["in_b"]), o_b=p(L["o_b"]),
+                 norm_w=p(L["norm1"]), norm_b=p(L["norm1b"]), ls1=p(L["ls1"]), canon=p(L["canon"]),
+                 inv_freq64=p(L["inv_freq64"]), q_norm=p(L.get("q_norm")), k_norm=p(L.get("k_norm")), qk_norm=int(m.qk_norm),
+                 sink=p(L.get("sink")), talk=p(L.get("talk")), v_from_k=int(m.v_from_k),
+                 **{"off_" + k: v for k, v in L["off"].items() if k in ("q", "k", "v", "g")})
+        if m.right is not None:
+            g = m.right
+            d.update(r_heads=g.heads, r_dim=g.dim, r_vdim=g.vdim, r_tau=g.tau, r_rank=g.decay_rank, off_rq=L["off"]["rq"],
+                     off_rk=L["off"]["rk"], off_rv=L["off"]["rv"], off_a1=L["off"]["a1"], a2=p(L["a2"]), a2_b=p(L["a2_b"]),
+                     gnorm=p(L["gnorm"]), w_o2=p(L["w_o2"]), left_scale=m.left_scale, right_scale=m.right_scale)
+        if f is not None:
+            if f.kind != FF_GLU:
+                raise ValueError("a sandwich layer's feed-forward is the gated dense one")
+            d.update(ff=f.ff, ff_dense=2, w_ff=p(L["w_ff"]), n_ff=L["n_ff"], w_dense_down=p(L["w_dense_down"]),
+                     norm2_w=p(L["norm2"]), norm2_b=p(L["norm2b"]), ls2=p(L["ls2"]))
+        return d
 
     def bind_chunks(self, rows) -> None:
         """The row tables of the next step: `rows` = (positions, sequence rows) of its B rows as the host
@@ -165,7 +192,12 @@ class StackRunner(Runner):
         self.kc, self.vc, self.states = [], [], []
         for li, _ps, _first in self.runs:
             m = cfg.layers[li].mixer
-            if m.kind == MIX_ATTENTION:
+            if cfg.block == BLOCK_SANDWICH:  # K/V pools, and one state row per slot: [second mixer's matrix | input window]
+                self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim, **tt))
+                self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
+                ns = cfg.run_state_floats(li)
+                self.states.append(torch.zeros(max_seqs, ns, **f32) if ns else None)
+            elif m.kind == MIX_ATTENTION:
                 self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim, **tt))
                 self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
                 self.states.append(None)
@@ -189,15 +221,19 @@ class StackRunner(Runner):
         self.catbuf = torch.zeros(max_batch, 2 * E, **tt)   # [x; x0], the pass-opening projection's operand
         n_proj = max(max(L["n_in"], L.get("n_ff", 0)) for L in self.w.layers)
         self.proj = torch.zeros(max_batch, (n_proj + 3) // 4 * 4, **f32)  # rows 16-byte aligned
-        self.abuf = torch.zeros(max_batch, max(s.mixer.n_out for s in cfg.layers), **tt)
-        self.hmid = torch.zeros(max_batch, (max([f.ff if f.kind == FF_DENSE else f.top * f.ff + f.shared_ff for f in mlps],
+        self.abuf = torch.zeros(max_batch, (max(s.mixer.n_out_all for s in cfg.layers) + 7) // 8 * 8, **tt)
+        self.hmid = torch.zeros(max_batch, (max([f.ff if f.kind in (FF_DENSE, FF_GLU) else f.top * f.ff + f.shared_ff for f in mlps],
                                                 default=1) + 7) // 8 * 8, **tt)
         # latent attention: queries folded onto the latent (float32), outputs in latent space (matrix dtype);
         # Mamba-2: the convolution's output (float32). idw: per-row weight of the chosen identity experts
         lat = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_LATENT]
         mam = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_MAMBA2]
-        self.cbuf = torch.zeros(max_batch, (max([m.heads * m.cache_dim for m in lat] + [m.conv_channels for m in mam],
-                                                default=1) + 3) // 4 * 4, **f32)
+        talk = [s.mixer for s in cfg.layers if s.mixer.talk]  # every query head against every key/value head's values
+        self.cbuf = torch.zeros(max_batch, (max([m.heads * m.cache_dim for m in lat] + [m.conv_channels for m in mam] +
+                                                [m.heads * m.kv_heads * m.vdim for m in talk], default=1) + 3) // 4 * 4, **f32)
+        sandwich = cfg.block == BLOCK_SANDWICH
+        self.hn = torch.zeros(max_batch if sandwich else 1, E, **f32)      # normed rows before the input convolution
+        self.ybuf2 = torch.zeros(max_batch if sandwich else 1, E, **f32)   # the second mixer's projected output
         self.latbuf = torch.zeros(max_batch, (max([m.heads * m.kv_rank for m in lat], default=1) + 7) // 8 * 8, **tt)
         self.idw = torch.zeros(max_batch, **f32)
         self.ybuf = torch.zeros(max_batch, E, **f32)
@@ -206,7 +242,9 @@ class StackRunner(Runner):
         self.sgate = torch.zeros(max_batch, **f32)
         self.lbuf = torch.zeros(max_batch, E, **tt)
         # state mixers' outputs before their norm (the mLSTM's with its normaliser's column per head)
-        self.obuf = torch.zeros(max_batch, max(s.mixer.heads * (s.mixer.vdim + (s.mixer.kind == MIX_MLSTM)) for s in cfg.layers), **f32)
+        self.obuf = torch.zeros(max_batch, max(max(s.mixer.heads * (s.mixer.vdim + (s.mixer.kind == MIX_MLSTM)),
+                                                   s.mixer.right.n_out if s.mixer.right is not None else 0)
+                                               for s in cfg.layers), **f32)
         # chunked retention of prompt portions: the chunk table and one state per chunk (its U, its incoming state)
         rets = [s.mixer for s in cfg.layers if s.mixer.kind in (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2)]
         n_ch = max_batch // 32 + max_seqs + 1 if rets and max_batch > 16 else 1
@@ -220,7 +258,8 @@ class StackRunner(Runner):
         self.scan_ctot = torch.zeros(n_ch, hmax, **f32) if hmax else None
         self.ret_sin = torch.zeros_like(self.ret_u)
         # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
-        hv = max([s.mixer.heads * (s.mixer.vdim + 2) for s in cfg.layers if s.mixer.kind == MIX_ATTENTION] +
+        hv = max([s.mixer.heads * (s.mixer.kv_heads if s.mixer.talk else 1) * (s.mixer.vdim + 2) for s in cfg.layers
+                  if s.mixer.kind == MIX_ATTENTION] +
                  [s.mixer.heads * (s.mixer.kv_rank + 2) for s in cfg.layers if s.mixer.kind == MIX_LATENT], default=1)
         self.split_ws = torch.zeros(16 * 16 * hv, **f32)
         self._step_rows = None  # (positions, sequence rows) of the rows last uploaded, until a step consumes them
@@ -282,6 +321,8 @@ class StackRunner(Runner):
         return S
 
     def _output_norm(self, h: torch.Tensor) -> torch.Tensor:
+        if self.w.final_b is None:
+            return h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.cfg.norm_eps) * self.w.final_w
         return torch.nn.functional.layer_norm(h, (h.shape[-1],), self.w.final_w, self.w.final_b, self.cfg.norm_eps)
 
     # ------------------------------------------------------------------ sequences and state slots

@@ -414,7 +414,7 @@ class StackWeights:
     def __init__(self, path: str, device: str | torch.device = "cuda", dtype: torch.dtype = torch.bfloat16):
         import os as _os
 
-        from ..models.config import BLOCK_POSTNORM, MIX_RETENTION, load_stack_config
+        from ..models.config import BLOCK_POSTNORM, BLOCK_SANDWICH, MIX_RETENTION, load_stack_config
         from .safetensors_io import SafetensorsFile
         self.cfg = cfg = self.full_cfg = load_stack_config(path)
         self.device, self.dtype = device, dtype
@@ -438,6 +438,9 @@ class StackWeights:
         for i, spec in enumerate(cfg.layers):
             m, f = spec.mixer, spec.mlp
             p = f"l{i}."
+            if cfg.block == BLOCK_SANDWICH:
+                self.layers.append(self._load_sandwich_layer(st, p, spec))
+                continue
             L: dict = dict(norm_w=vec(get(p + "norm1", (E,))), norm_b=vec(get(p + "norm1.b", (E,))))
             if cfg.block == BLOCK_POSTNORM:
                 self._load_postnorm_layer(L, p, spec)
@@ -476,7 +479,10 @@ class StackWeights:
             L["off"], L["n_in"] = off, n
             L["w_o"] = mat(get(p + "mix.o", (E, m.n_out)))
             self.layers.append(L)
-        self.final_w, self.final_b = vec(get("final.norm", (E,))), vec(get("final.norm.b", (E,)))
+        if cfg.block == BLOCK_SANDWICH:   # an RMS norm with one number as its weight
+            self.final_w, self.final_b = vec(get("final.norm", ())), None
+        else:
+            self.final_w, self.final_b = vec(get("final.norm", (E,))), vec(get("final.norm.b", (E,)))
         self.head = mat(get("head", (V, E)))
         self.local = dict(E=E, V=V)
 
@@ -545,6 +551,69 @@ class StackWeights:
             dn.append(get(q + "down", (E, F)))
         L["w_gu"] = mat(*gu).view(X, 2 * F, E)
         L["w_down"] = mat(*dn).view(X, E, F)
+
+    def _load_sandwich_layer(self, st, p: str, spec) -> dict:
+        """A layer with scalar-weight RMS norms around both sublayers. The matrices that read the mixer's input are
+        one stack `w_in` (attention q | k | [v], then a second mixer's q | k | v | gate | first decay factor) with
+        one float32 bias vector `in_b` over the stack (zero where a projection has none); the feed-forward's gate
+        and up rows are the stack `w_ff`. The inner size of the low-rank decay map comes from the tensor's shape.
+        Rotary frequencies are float64."""
+        from ..models.config import SINK_LEARNED, SINK_ONE, rotary_inv_freq
+        get, mat, vec = self._get, self._mat, self._vec
+        cfg, dev = self.cfg, self.device
+        E, m, f = cfg.n_embd, spec.mixer, spec.mlp
+        L: dict = {k: vec(get(p + k, ())) for k in ("norm1", "norm1b")}
+        L["ls1"] = vec(get(p + "ls1", (E,)))
+        L["canon"] = vec(get(p + "canon1", (E, cfg.canon_taps))) if cfg.canon_taps > 1 else None
+        a = p + ("mix.left." if m.right is not None else "mix.")
+        parts, off, bias, n = [], {}, [], 0
+
+        def add(key, name, rows, with_bias=False):
+            nonlocal n
+            parts.append(get(name, (rows, E)))
+            bias.append(get(name + ".b", (rows,)).to(torch.float32) if with_bias else torch.zeros(rows))
+            off[key] = n
+            n += rows
+
+        add("q", a + "q", m.n_q, m.bias)
+        add("k", a + "k", m.n_k, m.bias)
+        if m.v_from_k:
+            off["v"] = off["k"]
+        else:
+            add("v", a + "v", m.n_v, m.bias)
+        if m.qk_norm == 1:
+            L["q_norm"], L["k_norm"] = vec(get(a + "q.norm", (m.dim,))), vec(get(a + "k.norm", (m.dim,)))
+        if m.sink == SINK_LEARNED:
+            L["sink"] = vec(get(a + "sink", (m.heads,)))
+        elif m.sink == SINK_ONE:
+            L["sink"] = torch.zeros(m.heads, dtype=torch.float32, device=dev)
+        if m.talk:
+            L["talk"] = vec(get(a + "talk", (m.heads, m.heads)))
+        L["inv_freq64"] = (torch.tensor(rotary_inv_freq(m.rot_dims, m.rot_base, m.rot_scaling), dtype=torch.float64, device=dev)
+                           if m.rot_dims else None)
+        L["w_o"] = mat(get(a + "o", (E, m.n_out)))
+        L["o_b"] = vec(get(a + "o.b", (E,))) if m.o_bias else None
+        if m.right is not None:
+            r, b = m.right, p + "mix.right."
+            rank = st.shape(b + "a1")[0] if st.has(b + "a1") else 0
+            r.decay_rank = int(rank)
+            add("rq", b + "q", r.n_q)
+            add("rk", b + "k", r.n_q)
+            add("rv", b + "v", r.n_out)
+            add("g", b + "g", r.n_out)
+            add("a1", b + "a1", rank)
+            L["a2"] = mat(get(b + "a2", (r.n_q, rank)))
+            L["a2_b"] = vec(get(b + "a2.b", (r.n_q,)))
+            L["gnorm"] = vec(get(b + "norm", (r.vdim,)))
+            L["w_o2"] = mat(get(b + "o", (E, r.n_out)))
+        L["w_in"], L["in_b"] = mat(*parts), torch.cat(bias).contiguous().to(dev)
+        L["off"], L["n_in"], L["n_ff"] = off, n, 0
+        if f is not None:
+            L.update({k: vec(get(p + k, ())) for k in ("norm2", "norm2b")})
+            L["ls2"] = vec(get(p + "ls2", (E,)))
+            L["w_ff"], L["n_ff"] = mat(get(p + "mlp.gate", (f.ff, E)), get(p + "mlp.up", (f.ff, E))), 2 * f.ff
+            L["w_dense_down"] = mat(get(p + "mlp.down", (E, f.ff)))
+        return L
 
     @property
     def nbytes(self) -> int:

@@ -249,16 +249,53 @@ MIX_RETENTION = 1   # decayed linear attention with a per-sequence state matrix
 MIX_LATENT = 2      # softmax attention whose keys and values come from one cached low-rank latent per token
 MIX_MLSTM = 3       # matrix memory with exponential input / forget gates and a running stabiliser
 MIX_MAMBA2 = 4      # selective state space layer (scalar decay per head) behind a short causal convolution
-STATE_MIXERS = (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2)   # mixers that own a per-sequence state slot
+MIX_GLA = 5         # gated linear attention: a state matrix whose rows (key channels) decay by a per-token vector
+STATE_MIXERS = (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2, MIX_GLA)   # mixers that own a per-sequence state slot
 
 BLOCK_PARALLEL = 0  # x <- x + m (mixer(LN(x)) + ff(LN(x))): one norm, both sublayers read it
 BLOCK_POSTNORM = 1  # x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)): the norm sits on the sublayer's output
+BLOCK_SANDWICH = 2  # x <- x + s1 N1b(mixer(conv_in(N1(x)))), then x <- x + s2 N2b(ff(N2(x))): scalar-weight RMS norms
+                    # before and after each sublayer, per-channel scales on the results, a short causal convolution
+                    # added to the mixer's input
 
 FF_MOE = 0          # routed experts (+ shared expert)
 FF_DENSE = 1        # W_down act(W_up h), act = relu(z)^2
+FF_GLU = 2          # W_down (act(W_gate h) * (W_up h)), act = the tanh form of gelu
 ROUTE_TOPK_SOFTMAX = 0   # top-k of (logits + bias), softmax over the chosen logits
 ROUTE_SCORE_GROUPS = 1   # softmax over all outputs; choice by score + correction inside the best expert groups;
                          # weights = the chosen scores; trailing outputs may be identity experts
+
+
+QK_NORM_NONE = 0
+QK_NORM_WEIGHT_FIRST = 1    # RMS norm with a [dim] weight shared by the heads, before the rotation
+QK_NORM_UNIT_LAST = 2       # division by the root mean square (no weight), after the rotation
+SINK_NONE = 0
+SINK_LEARNED = 1            # exp(sink_h), a learned number per head, joins the softmax denominator
+SINK_ONE = 2                # a sink of score 0: the denominator holds one extra 1
+
+
+def rotary_inv_freq(dims: int, base: float, scaling: tuple = ()) -> list:
+    """Rotary frequencies f_i = base^(-2i / dims), i < dims / 2, in float64, with the scaling a config names."""
+    import math
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    if not scaling:
+        return f
+    if scaling[0] == "linear":
+        return [x / float(scaling[1]) for x in f]
+    if scaling[0] != "bands":
+        raise UnsupportedArchitecture(f"unknown rotary scaling {scaling[0]!r}")
+    _, factor, low, high, original = scaling
+    out = []
+    for x in f:
+        wave = 2.0 * math.pi / x
+        if wave < original / high:
+            out.append(x)
+        elif wave > original / low:
+            out.append(x / factor)
+        else:
+            t = (original / wave - low) / (high - low)
+            out.append((1.0 - t) * x / factor + t * x)
+    return out
 
 
 @dataclass
@@ -289,6 +326,22 @@ class MixerSpec:
     groups: int = 1
     conv: int = 1               # taps of the causal convolution (the last one is the current token's)
     norm_groups: int = 1        # the gated output is RMS-normed in this many equal parts
+    # attention options of the sandwich block's mixers
+    bias: bool = False          # q, k, v (and with o_bias the output) projections carry biases
+    o_bias: bool = False
+    rot_scaling: tuple = ()     # () none; ("linear", factor); ("bands", factor, low, high, original): long waves
+                                # divided by factor, short ones kept, a linear blend between
+    qk_norm: int = QK_NORM_NONE
+    sink: int = SINK_NONE
+    talk: bool = False          # the heads' softmax weights are mixed by a [heads, heads] matrix before the values
+    v_from_k: bool = False      # the values are the projected keys (before norm and rotation); no value projection
+    # gated linear attention
+    tau: float = 1.0            # decay = sigmoid(z)^(1 / tau)
+    decay_rank: int = 0         # inner size of the low-rank map that gives z (read from the tensor's shape)
+    # a second mixer that reads the same input; the layer's result is left_scale * this + right_scale * right
+    right: "MixerSpec | None" = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
 
     @property
     def n_q(self) -> int:
@@ -307,6 +360,10 @@ class MixerSpec:
         return self.heads * self.vdim
 
     @property
+    def n_out_all(self) -> int:  # with the second mixer's beside it
+        return self.n_out + (self.right.n_out if self.right is not None else 0)
+
+    @property
     def conv_channels(self) -> int:   # mamba2: x | B | C pass the convolution
         return self.heads * self.vdim + 2 * self.groups * self.state
 
@@ -317,7 +374,7 @@ class MixerSpec:
     @property
     def state_floats(self) -> int:
         """float32 words of the per-sequence state of one run of this mixer."""
-        if self.kind == MIX_RETENTION:
+        if self.kind in (MIX_RETENTION, MIX_GLA):
             return self.heads * self.dim * self.vdim
         if self.kind == MIX_MLSTM:      # S [H][dim][vdim] | n [H][dim] | m [H]
             return self.heads * (self.dim * self.vdim + self.dim + 1)
@@ -364,6 +421,8 @@ class StackConfig:
     logit_softcap: float = 0.0
     block: int = BLOCK_PARALLEL
     embed_scale: float = 1.0
+    logit_scale: float = 1.0    # logits = head x * logit_scale
+    canon_taps: int = 1         # sandwich block: taps of the convolution added to the mixer's input (1 = none)
     ctx_len: int = 1 << 20      # the design has no positional table: bounded by the cache pool only
     bos_id: int = 0
     eos_id: int = -1            # no tokenizer ships with these models: generation never stops on a token
@@ -390,7 +449,16 @@ class StackConfig:
     @property
     def has_state(self) -> bool:
         """Some layer carries a recurrent state: a cached prefix cannot be cut back to an earlier length."""
-        return any(s.mixer.kind in STATE_MIXERS for s in self.layers)
+        return self.canon_taps > 1 or any(s.mixer.kind in STATE_MIXERS or s.mixer.right is not None for s in self.layers)
+
+    def run_state_floats(self, li: int) -> int:
+        """float32 words of the per-sequence state of one run of layer li: the mixer's (and its second mixer's) state
+        matrix, then, in a sandwich block, the last canon_taps - 1 inputs of the input convolution."""
+        m = self.layers[li].mixer
+        n = m.state_floats + (m.right.state_floats if m.right is not None else 0)
+        if self.block == BLOCK_SANDWICH:
+            n += (self.canon_taps - 1) * self.n_embd
+        return n
 
     def to_dict(self) -> dict:
         return asdict(self)
@@ -562,11 +630,103 @@ class StackConfig:
         return dict(architecture="Norevik", vocab=self.n_vocab, width=self.n_embd, layers=out,
                     norm=dict(eps=self.norm_eps), embedding=dict(scale=self.embed_scale))
 
+    # -- config.json of the Suvunex design
+    @classmethod
+    def from_suvunex(cls, c: dict) -> "StackConfig":
+        def bad(msg):
+            raise UnsupportedArchitecture("Suvunex: " + msg)
+
+        def attention(m: dict, **kw) -> MixerSpec:
+            rot = m.get("rot") or {}
+            sc = rot.get("scaling") or {}
+            if not sc:
+                scaling = ()
+            elif "original" in sc:
+                scaling = ("bands", float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
+                if scaling[3] == scaling[2]:
+                    bad("rot.scaling: high and low must differ")
+            else:
+                scaling = ("linear", float(sc["factor"]))
+            mx = MixerSpec(kind=MIX_ATTENTION, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                           dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                           rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), rot_scaling=scaling,
+                           bias=True, **kw)
+            if mx.rot_dims % 2 or mx.rot_dims > mx.dim:
+                bad("rot.dims must be even and at most dim")
+            if min(mx.heads, mx.kv_heads, mx.dim, mx.vdim) <= 0 or mx.heads % mx.kv_heads:
+                bad("heads must be a positive multiple of kv_heads")
+            return mx
+
+        layers = []
+        for ent in c["layers"]:
+            m, t = ent["mixer"], ent["type"]
+            if t == "parallel":
+                mx = attention(m["left"], o_bias=True, qk_norm=QK_NORM_UNIT_LAST, sink=SINK_ONE)
+                r = m["right"]
+                mx.right = MixerSpec(kind=MIX_GLA, heads=int(r["heads"]), kv_heads=int(r["heads"]), dim=int(r["dim"]),
+                                     vdim=int(r["vdim"]), tau=float(r["tau"]))
+                if min(mx.right.heads, mx.right.dim, mx.right.vdim) <= 0 or mx.right.tau <= 0:
+                    bad("right: sizes and tau must be positive")
+                mx.left_scale, mx.right_scale = float(m["left_scale"]), float(m["right_scale"])
+            elif t == "attention":
+                mx = attention(m, qk_norm=QK_NORM_WEIGHT_FIRST, sink=SINK_LEARNED, talk=True, v_from_k=True)
+                if mx.vdim != mx.dim:
+                    bad("attention: the values are the keys, so vdim must equal dim")
+            else:
+                raise UnsupportedArchitecture(f"unknown mixer type {t!r}")
+            mlp = None
+            f = ent.get("mlp")
+            if f:
+                if f.get("kind") != "dense":
+                    raise UnsupportedArchitecture(f"unknown feed-forward kind {f.get('kind')!r}")
+                mlp = MoESpec(kind=FF_GLU, ff=int(f["ff"]))
+                if mlp.ff <= 0:
+                    bad("mlp.ff must be positive")
+            layers.append(LayerSpec(mixer=mx, mlp=mlp))
+        taps = int((c.get("canon") or {}).get("taps", 1))
+        if taps < 1:
+            bad("canon.taps must be at least 1")
+        return cls(arch="suvunex", n_vocab=int(c["vocab"]), n_embd=int(c["width"]), layers=layers,
+                   norm_eps=float(c["norm"]["eps"]), block=BLOCK_SANDWICH, canon_taps=taps,
+                   embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                   logit_scale=float(c.get("logit_scale", 1.0)), name=str(c.get("name", "")))
+
+    def to_suvunex(self) -> dict:
+        """The config.json this configuration is read from (random-init fixtures, tests)."""
+        def attention(m: MixerSpec) -> dict:
+            d = dict(heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale)
+            if m.rot_dims:
+                d["rot"] = dict(base=m.rot_base, dims=m.rot_dims)
+                if m.rot_scaling and m.rot_scaling[0] == "linear":
+                    d["rot"]["scaling"] = dict(factor=m.rot_scaling[1])
+                elif m.rot_scaling:
+                    _, fa, lo, hi, orig = m.rot_scaling
+                    d["rot"]["scaling"] = dict(factor=fa, low=lo, high=hi, original=orig)
+            return d
+
+        out = []
+        for s in self.layers:
+            m = s.mixer
+            if m.right is not None:
+                r = m.right
+                ent = dict(type="parallel", mixer=dict(left=attention(m), left_scale=m.left_scale, right_scale=m.right_scale,
+                                                       right=dict(heads=r.heads, dim=r.dim, vdim=r.vdim, tau=r.tau)))
+            elif m.kind == MIX_ATTENTION and m.talk:
+                ent = dict(type="attention", mixer=attention(m))
+            else:
+                raise UnsupportedArchitecture("Suvunex has no mixer of this kind")
+            ent["mlp"] = None if s.mlp is None else dict(kind="dense", ff=s.mlp.ff)
+            out.append(ent)
+        return dict(architecture="Suvunex", vocab=self.n_vocab, width=self.n_embd, layers=out, norm=dict(eps=self.norm_eps),
+                    embedding=dict(scale=self.embed_scale), canon=dict(taps=self.canon_taps), logit_scale=self.logit_scale)
+
     def to_config_json(self) -> dict:
+        if self.arch == "suvunex":
+            return self.to_suvunex()
         return self.to_norevik() if self.arch == "norevik" else self.to_bizulix()
 
 
-STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix, "Norevik": StackConfig.from_norevik}
+STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix, "Norevik": StackConfig.from_norevik, "Suvunex": StackConfig.from_suvunex}
 
 
 def is_stack_model(path: str) -> bool:

@@ -382,6 +382,101 @@ def stack_route_scores(z, corr, top, n_real, group_count, group_keep):
     return torch.where(ident, 0, ids).to(torch.int32), torch.where(ident, 0.0, wt), idw
 
 
+
+# ---- layers with scalar-weight RMS norms around both sublayers (BLOCK_SANDWICH): an input convolution with a
+# carried window, attention with biases / rotation with scaled frequencies / query and key norms / sinks / mixing of
+# the heads' weights, gated linear attention beside it, a gated feed-forward. One function per kernel of
+# csrc/stack/stack_sandwich.hip.
+
+def stack_scalar_norm(x, g, eps):
+    """x / sqrt(mean(x^2) + eps) * g with one number g for all coordinates."""
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * g
+
+
+def stack_canon_conv(hn, w, window, q_seq):
+    """hn [B, E] + causal per-channel convolution over each sequence's rows (w [E, taps], the last tap is the
+    current token's), continued from `window` [slots, taps - 1, E] (the sequence's last inputs, oldest first),
+    which is advanced in place."""
+    B, K = hn.shape[0], w.shape[1]
+    out = torch.empty_like(hn)
+    for b in range(B):
+        st = window[int(q_seq[b])]
+        win = torch.cat([st, hn[b:b + 1]], 0)                  # [K, E]
+        out[b] = hn[b] + (win * w.T).sum(0)
+        if K > 1:
+            st.copy_(win[1:])
+    return out
+
+
+def stack_rotate_half64(x, pos, inv_freq):
+    """x [B, H, D] float32: dims i and i + n (n = len(inv_freq)) turn by pos * inv_freq[i]; float64 angles."""
+    n = inv_freq.numel()
+    ang = pos.double()[:, None] * inv_freq.double()[None, :]
+    c, s = torch.cos(ang).float()[:, None, :], torch.sin(ang).float()[:, None, :]
+    u, v = x[..., :n], x[..., n:2 * n]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., 2 * n:]], -1)
+
+
+def stack_qk_prepare(q, k, m, L, pos, eps):
+    """Queries [B, H, D] and keys [B, G, D] (biases added): RMS norm with a weight before the rotation, or unit RMS
+    after it, as the mixer says."""
+    def unit(t):
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+    if m.qk_norm == 1:
+        q, k = unit(q) * L["q_norm"], unit(k) * L["k_norm"]
+    if m.rot_dims:
+        q, k = stack_rotate_half64(q, pos, L["inv_freq64"]), stack_rotate_half64(k, pos, L["inv_freq64"])
+    if m.qk_norm == 2:
+        q, k = unit(q), unit(k)
+    return q, k
+
+
+def stack_attention_sink(q, kc, vc, block_table, q_seq, q_len, bs, scale, groups, sink, talk):
+    """Softmax attention over the paged pools with exp(sink_h) in the denominator (sink None: none). With `talk`
+    [H, H] the heads' weights are mixed, w_h <- sum_g talk[h, g] w_g, before head h meets the values of its own
+    key/value head. Returns float32 [B, H, Dv]."""
+    B, H, _ = q.shape
+    out = torch.empty(B, H, vc.shape[-1], dtype=torch.float32, device=q.device)
+    for b in range(B):
+        n = int(q_len[b])
+        t = torch.arange(n, device=q.device)
+        bt = block_table[int(q_seq[b])].long()
+        kk = kc[bt[t // bs], :, t % bs].float().repeat_interleave(groups, dim=1)  # [n, H, D]
+        vv = vc[bt[t // bs], :, t % bs].float().repeat_interleave(groups, dim=1)
+        s = torch.einsum("hd,thd->ht", q[b], kk) * scale
+        mx = s.max(-1, keepdim=True).values
+        if sink is not None:
+            mx = torch.maximum(mx, sink[:, None])
+        e = torch.exp(s - mx)
+        den = e.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sink[:, None] - mx)
+        w = e / den
+        if talk is not None:
+            w = talk @ w
+        out[b] = torch.einsum("ht,thd->hd", w, vv)
+    return out
+
+
+def stack_gla(q, k, v, alpha, S, q_seq):
+    """S [slots, H, D, Dv] <- diag(alpha) S + k v^T per row (alpha [B, H, D]), o = S^T q. Returns float32 [B, H, Dv]."""
+    out = torch.empty_like(v)
+    for r in range(q.shape[0]):
+        St = S[int(q_seq[r])]
+        St.mul_(alpha[r][:, :, None]).add_(k[r][:, :, None] * v[r][:, None, :])
+        out[r] = torch.einsum("hdv,hd->hv", St, q[r])
+    return out
+
+
+def stack_gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+
+
+def stack_sandwich_add(x, y, g, ls, eps):
+    """x += ls * (y / rms(y) * g): the scalar-weight norm on a sublayer's result, then the per-channel scale."""
+    x += ls * stack_scalar_norm(y, g, eps)
+
+
 class TorchStackExecutor:
     def __init__(self, runner):
         self.r = runner
@@ -393,11 +488,13 @@ class TorchStackExecutor:
         r.x0[:B] = x
 
     def layer_run(self, ri: int, B: int):
-        from ..models.config import BLOCK_POSTNORM, MIX_ATTENTION
+        from ..models.config import BLOCK_POSTNORM, BLOCK_SANDWICH, MIX_ATTENTION
         r = self.r
         w, cfg, T = r.w, r.cfg, r.w.dtype
         if cfg.block == BLOCK_POSTNORM:
             return self.layer_run_postnorm(ri, B)
+        if cfg.block == BLOCK_SANDWICH:
+            return self.layer_run_sandwich(ri, B)
         li, _ps, opens = r.runs[ri]
         L, spec = w.layers[li], cfg.layers[li]
         m, f, off = spec.mixer, spec.mlp, L["off"]
@@ -534,12 +631,74 @@ class TorchStackExecutor:
         r.ybuf[:B] = y
         stack_post_norm_add(x, r.ybuf[:B], L["norm2_w"], L["norm2_b"], cfg.norm_eps, idw)
 
+    def layer_run_sandwich(self, ri: int, B: int):
+        """x <- x + s1 N1b(mixer(conv_in(N1(x)))), then x <- x + s2 N2b(ff(N2(x)))."""
+        r = self.r
+        w, cfg, T = r.w, r.cfg, r.w.dtype
+        li = r.runs[ri][0]
+        L, spec = w.layers[li], cfg.layers[li]
+        m, f, off, E, eps = spec.mixer, spec.mlp, L["off"], cfg.n_embd, cfg.norm_eps
+        x = r.resid[:B]
+        pos, qseq = r.d_pos[:B], r.d_qseq[:B]
+        st = r.states[ri]
+        hn = stack_scalar_norm(x, L["norm1"], eps)
+        r.hn[:B] = hn
+        if cfg.canon_taps > 1:
+            nS = st.shape[1] - (cfg.canon_taps - 1) * E
+            hn = stack_canon_conv(hn, L["canon"].view(E, cfg.canon_taps), st[:, nS:].view(st.shape[0], cfg.canon_taps - 1, E), qseq)
+        r.hbuf[:B] = hn.to(T)
+        proj = stack_matmul(r.hbuf[:B], L["w_in"])
+        r.proj[:B, :proj.shape[1]] = proj
+        H, G, D, Dv = m.heads, m.kv_heads, m.dim, m.vdim
+        bias = L["in_b"]
+        q = (proj[:, off["q"]:off["q"] + H * D] + bias[off["q"]:off["q"] + H * D]).view(B, H, D)
+        k = (proj[:, off["k"]:off["k"] + G * D] + bias[off["k"]:off["k"] + G * D]).view(B, G, D)
+        v = k if m.v_from_k else (proj[:, off["v"]:off["v"] + G * Dv] + bias[off["v"]:off["v"] + G * Dv]).view(B, G, Dv)
+        q, kk = stack_qk_prepare(q, k, m, L, pos, eps)
+        slot = r.d_slot[:B].long()
+        blk, o = slot // r.block_size, slot % r.block_size
+        r.kc[ri][blk, :, o] = kk.to(T)
+        r.vc[ri][blk, :, o] = v.to(T)
+        a = stack_attention_sink(q, r.kc[ri], r.vc[ri], r.d_block_table, qseq, r.d_qlen[:B], r.block_size, m.scale, H // G,
+                                 L.get("sink"), L["talk"].view(H, H) if m.talk else None)
+        n1 = m.n_out
+        r.abuf[:B, :n1] = a.reshape(B, n1).to(T)
+        y = stack_matmul(r.abuf[:B, :n1], L["w_o"])
+        if L["o_b"] is not None:
+            y = y + L["o_b"]
+        if m.right is not None:
+            g = m.right
+            Hr, Dr, Dvr, n2 = g.heads, g.dim, g.vdim, g.n_out
+            rq = proj[:, off["rq"]:off["rq"] + Hr * Dr].view(B, Hr, Dr) * float(Dr) ** -0.5
+            rk = proj[:, off["rk"]:off["rk"] + Hr * Dr].view(B, Hr, Dr)
+            rv = proj[:, off["rv"]:off["rv"] + n2].view(B, Hr, Dvr)
+            z = proj[:, off["a1"]:off["a1"] + g.decay_rank] @ L["a2"].float().T + L["a2_b"]
+            alpha = torch.exp(F.logsigmoid(z) / g.tau).view(B, Hr, Dr)
+            S = st[:, :Hr * Dr * Dvr].view(-1, Hr, Dr, Dvr)
+            o2 = stack_gla(rq, rk, rv, alpha, S, qseq)
+            o2 = o2 * torch.rsqrt(o2.pow(2).mean(-1, keepdim=True) + eps) * L["gnorm"]
+            r.abuf[:B, n1:n1 + n2] = (o2.reshape(B, n2) * F.silu(proj[:, off["g"]:off["g"] + n2])).to(T)
+            y = m.left_scale * y + m.right_scale * stack_matmul(r.abuf[:B, n1:n1 + n2], L["w_o2"])
+        stack_sandwich_add(x, y, L["norm1b"], L["ls1"], eps)
+        if f is None:
+            return
+        r.hbuf[:B] = stack_scalar_norm(x, L["norm2"], eps).to(T)
+        proj = stack_matmul(r.hbuf[:B], L["w_ff"])
+        r.proj[:B, :proj.shape[1]] = proj
+        r.hmid[:B, :f.ff] = (stack_gelu_tanh(proj[:, :f.ff]) * proj[:, f.ff:2 * f.ff]).to(T)
+        stack_sandwich_add(x, stack_matmul(r.hmid[:B, :f.ff], L["w_dense_down"]), L["norm2b"], L["ls2"], eps)
+
     def head(self, n_logits: int, use_idx: bool):
         r = self.r
         if n_logits <= 0:
             return
         w, cfg = r.w, r.cfg
         x = r.resid[r.d_logit_idx[:n_logits].long()] if use_idx else r.resid[:n_logits]
+        if w.final_b is None:  # an RMS norm with one number as its weight, and a plain factor on the logits
+            r.lbuf[:n_logits] = stack_scalar_norm(x, w.final_w, cfg.norm_eps).to(w.dtype)
+            z = stack_matmul(r.lbuf[:n_logits], w.head) * float(cfg.logit_scale)
+            r.logits[:n_logits, :z.shape[1]] = z
+            return
         r.lbuf[:n_logits] = F.layer_norm(x, (x.shape[-1],), w.final_w, w.final_b, cfg.norm_eps).to(w.dtype)
         z = stack_matmul(r.lbuf[:n_logits], w.head)
         if cfg.logit_softcap:
