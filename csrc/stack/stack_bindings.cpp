@@ -50,6 +50,8 @@ PYBIND11_MODULE(_stack, m) {
   m.def("retention_supported", &retention_supported);
   m.def("gated_scan_supported", &gated_scan_supported);
   m.def("latent_supported", &latent_supported);
+  m.def("gla_supported", &gla_supported);
+  m.def("gla_chunk_supported", &gla_chunk_supported);
   m.def("gated_chunk_rows", &gated_chunk_rows);
   m.def("retention_chunk_rows", &retention_chunk_rows);
   m.attr("FLASH_TILE_ROWS") = (int)FLASH_TILE_ROWS;
@@ -67,6 +69,8 @@ PYBIND11_MODULE(_stack, m) {
         e.cfg.max_seqs = geti(c, "max_seqs");
         e.cfg.block = geti(c, "block");
         e.cfg.embed_scale = getf(c, "embed_scale", 1.f);
+        e.cfg.logit_scale = getf(c, "logit_scale", 1.f);
+        e.cfg.canon_taps = geti(c, "canon_taps", 1);
       })
       .def("set_globals", [](StackExecutor& e, py::dict d) {
         e.embed_w = Pp<const void>(ptr(d, "embed"));
@@ -148,6 +152,31 @@ PYBIND11_MODULE(_stack, m) {
         L.dt_bias = Pp<const float>(ptr(d, "dt_bias"));
         L.a_log = Pp<const float>(ptr(d, "a_log"));
         L.d_skip = Pp<const float>(ptr(d, "d_skip"));
+        L.in_b = Pp<const float>(ptr(d, "in_b"));
+        L.o_b = Pp<const float>(ptr(d, "o_b"));
+        L.ls1 = Pp<const float>(ptr(d, "ls1"));
+        L.ls2 = Pp<const float>(ptr(d, "ls2"));
+        L.canon = Pp<const float>(ptr(d, "canon"));
+        L.qk_norm = geti(d, "qk_norm");
+        L.v_from_k = geti(d, "v_from_k");
+        L.q_norm = Pp<const float>(ptr(d, "q_norm"));
+        L.k_norm = Pp<const float>(ptr(d, "k_norm"));
+        L.talk = Pp<const float>(ptr(d, "talk"));
+        L.r_heads = geti(d, "r_heads");
+        L.r_dim = geti(d, "r_dim");
+        L.r_vdim = geti(d, "r_vdim");
+        L.r_rank = geti(d, "r_rank");
+        L.r_tau = getf(d, "r_tau", 1.f);
+        L.left_scale = getf(d, "left_scale", 1.f);
+        L.right_scale = getf(d, "right_scale", 1.f);
+        L.off_rq = geti(d, "off_rq");
+        L.off_rk = geti(d, "off_rk");
+        L.off_rv = geti(d, "off_rv");
+        L.off_a1 = geti(d, "off_a1");
+        L.a2 = Pp<const void>(ptr(d, "a2"));
+        L.a2_b = Pp<const float>(ptr(d, "a2_b"));
+        L.gnorm = Pp<const float>(ptr(d, "gnorm"));
+        L.w_o2 = Pp<const void>(ptr(d, "w_o2"));
         if (L.qtemp_every <= 0) throw std::runtime_error("q_temp.every must be positive");
       })
       .def("set_runs", [](StackExecutor& e, std::vector<py::dict> runs) {
@@ -208,6 +237,9 @@ PYBIND11_MODULE(_stack, m) {
         w.coef = Pp<float>(ptr(d, "coef"));
         w.ld_coef = geti(d, "ld_coef");
         w.ctot = Pp<float>(ptr(d, "ctot"));
+        w.hn = Pp<float>(ptr(d, "hn"));
+        w.y2 = Pp<float>(ptr(d, "y2"));
+        w.lna = w.coef;
       })
       .def("set_inputs", [](StackExecutor& e, py::dict d) {
         StackInputs& in = e.in;

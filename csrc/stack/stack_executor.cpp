@@ -42,15 +42,47 @@ static void validate_postnorm(const StackExecutor& e, const RunDesc& r, const La
   }
 }
 
+static void validate_sandwich(const StackExecutor& e, const RunDesc& r, const LayerDesc& L) {
+  const StackWorkspace& ws = e.ws;
+  const int taps = e.cfg.canon_taps;
+  need(L.kind == 0 && r.kc && r.vc, "a layer with scalar norms needs an attention mixer with K/V pools");
+  need(L.norm_w && L.norm_b && L.ls1 && L.w_in && L.w_o && L.n_in > 0 && L.n_in <= ws.ld_proj && ws.hn && ws.y2,
+       "layer weights or buffers missing");
+  need(L.dim <= 256 && L.vdim <= 256 && L.kv_heads > 0 && L.heads % L.kv_heads == 0, "attention head sizes");
+  need(L.rot_dims % 2 == 0 && L.rot_dims <= L.dim && (L.rot_dims == 0 || L.inv_freq64), "rotary table missing");
+  need(L.qk_norm != QK_NORM_WEIGHT_FIRST || (L.q_norm && L.k_norm), "query / key norm weights missing");
+  need(!L.v_from_k || L.vdim == L.dim, "values that are the keys need vdim == dim");
+  need(!L.talk || (ws.cbuf && (long long)L.heads * L.kv_heads * L.vdim <= ws.ld_cbuf), "mixed heads: float32 buffer too small");
+  need(taps >= 1 && taps <= CANON_MAX_TAPS && (taps == 1 || (L.canon && r.state)), "input convolution (1..8 taps) operands");
+  long long need_state = (long long)(taps - 1) * e.cfg.E;
+  int n_out = L.heads * L.vdim;
+  if (L.r_heads) {
+    need(L.a2 && L.a2_b && L.gnorm && L.w_o2 && L.r_rank > 0 && L.r_tau > 0.f && r.state, "gated linear attention operands");
+    need(gla_supported(L.r_dim, L.r_vdim), "gated linear attention head sizes (<= 256, state within the registers)");
+    need_state += (long long)L.r_heads * L.r_dim * L.r_vdim;
+    n_out += L.r_heads * L.r_vdim;
+  }
+  need(r.state_stride >= need_state, "state slot too small");
+  need(n_out <= ws.ld_a, "mixer output wider than its buffer");
+  if (L.ff_dense)
+    need(L.ff_dense == 2 && L.w_ff && L.w_dense_down && L.norm2_w && L.norm2_b && L.ls2 && L.ff > 0 && L.ff <= ws.ld_hmid &&
+             2 * L.ff <= ws.ld_proj && ws.hmid,
+         "gated feed-forward operands");
+}
+
 void StackExecutor::validate() const {
   need(cfg.E > 0 && cfg.V > 0 && cfg.max_B > 0, "not configured");
-  need(embed_w && final_w && final_b && head_w, "global weights missing");
+  need(embed_w && final_w && (final_b || cfg.block == 2) && head_w, "global weights missing");
   need(ws.resid && ws.x0 && ws.h && ws.proj && ws.a && ws.y && ws.lrows, "workspace missing");
   need(in.tokens && in.pos && in.slot && in.q_len && in.q_seq && in.block_table && in.logits, "step inputs missing");
   need(!runs.empty(), "no layer runs");
   for (const RunDesc& r : runs) {
     need(r.layer >= 0 && r.layer < (int)layers.size(), "a run names a layer that does not exist");
     const LayerDesc& L = layers[r.layer];
+    if (cfg.block == 2) {
+      validate_sandwich(*this, r, L);
+      continue;
+    }
     need(L.norm_w && L.norm_b && L.w_in && L.w_o && L.n_in > 0 && L.n_in <= ws.ld_proj, "layer weights missing");
     need(L.heads * L.vdim <= ws.ld_a, "mixer output wider than its buffer");
     if (cfg.block == 1) {
@@ -217,9 +249,84 @@ void StackExecutor::layer_run_postnorm(int ri, int B, hipStream_t s) {
   post_norm_add(ws.resid, ws.y, B, E, L.norm2_w, L.norm2_b, cfg.eps, idw, ws.h, f32, s);
 }
 
+// x <- x + s1 N1b(mixer(conv_in(N1(x)))), then x <- x + s2 N2b(ff(N2(x))); N: RMS norm with one number as weight.
+// The mixer is softmax attention (biases, rotation, query / key norms, a sink, optionally mixed heads and values that
+// are the keys), optionally with a gated linear attention beside it that reads the same input.
+void StackExecutor::layer_run_sandwich(int ri, int B, hipStream_t s) {
+  const RunDesc& r = runs.at(ri);
+  const LayerDesc& L = layers[r.layer];
+  const int E = cfg.E, f32 = cfg.f32, taps = cfg.canon_taps;
+  const int n1 = L.heads * L.vdim, n2 = L.r_heads * L.r_vdim;
+  const long long gla_floats = (long long)L.r_heads * L.r_dim * L.r_vdim;  // the slot: [state matrix | input window]
+  StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
+  {
+    CanonParams C{ws.resid, L.norm_w, cfg.eps, E, taps, L.canon, r.state ? r.state + gla_floats : nullptr, r.state_stride, ws.hn, ws.h,
+                  f32};
+    scalar_norm_conv(C, R, s);
+  }
+  {  // every matrix that reads the mixer's input, in one product
+    GemmParams g{ws.h, E, L.w_in, B, L.n_in, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  {
+    QkPrepParams Q{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.in_b, L.heads, L.kv_heads, L.dim, L.vdim, L.rot_dims,
+                   L.inv_freq64, L.qk_norm, L.q_norm, L.k_norm, cfg.eps, L.v_from_k, r.kc, r.vc, f32};
+    qk_prepare(Q, R, s);
+    AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, 0.f, 0.f, 1, r.kc, r.vc,
+                 ws.a, ws.ld_a, f32, n_splits, ws.split_ws, ws.split_ws_floats, 0, 0, L.sink, 0, nullptr, 0};
+    if (L.talk) {  // every query head's weights on every key/value head's values, in float32; then the heads are mixed
+      A.vheads = L.kv_heads;
+      A.out32 = ws.cbuf;
+      A.ld_out32 = ws.ld_cbuf;
+    }
+    if (B > SMALL_B && n_tiles > 0 && tiles && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);  // prompt portions: query tiles on the matrix cores
+    else
+      attention(A, R, s);
+    if (L.talk) talk_mix(ws.cbuf, ws.ld_cbuf, B, L.heads, L.kv_heads, L.vdim, L.talk, ws.a, ws.ld_a, f32, s);
+  }
+  {
+    GemmParams o{ws.a, ws.ld_a, L.w_o, B, E, n1, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(o, s);
+  }
+  if (L.r_heads) {
+    const size_t esz = f32 ? 4 : 2;
+    GlaParams G{ws.proj, ws.ld_proj, L.off_rq, L.off_rk, L.off_rv, L.off_g, L.off_a1, L.r_heads, L.r_dim, L.r_vdim, L.r_rank, L.a2,
+                L.a2_b, L.r_tau, L.gnorm, cfg.eps, r.state, r.state_stride, (char*)ws.a + (size_t)n1 * esz, ws.ld_a, f32};
+    if (B > SMALL_B && n_chunks > 0 && ws.ret.U && ws.ret.Sin && ws.lna && ws.ld_coef >= L.r_heads * L.r_dim &&
+        ws.ret.u_stride >= gla_floats && gla_chunk_supported(L.r_dim, L.r_vdim)) {
+      GlaChunkWs W{ws.ret.chunks, n_chunks, ws.ret.max_chunks, ws.ret.U, ws.ret.Sin, ws.ret.u_stride, ws.lna, ws.ld_coef, nullptr, 0};
+      gla_chunked(G, R, W, s);  // prompt portions: chunks in parallel around a scan over the chunk states
+    } else {
+      gla(G, R, s);
+    }
+    GemmParams o{(char*)ws.a + (size_t)n1 * esz, ws.ld_a, L.w_o2, B, E, n2, ws.y2, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(o, s);
+  }
+  const bool has_ff = L.ff_dense != 0;
+  // the updated rows leave normed for the feed-forward in the same launch
+  sandwich_add(ws.resid, ws.y, L.o_b, L.r_heads ? L.left_scale : 1.f, L.r_heads ? ws.y2 : nullptr, L.right_scale, B, E, L.norm_b,
+               L.ls1, cfg.eps, has_ff ? L.norm2_w : nullptr, has_ff ? ws.h : nullptr, f32, s);
+  if (!has_ff) return;
+  {
+    GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  geglu_tanh_cast(ws.proj, ws.ld_proj, B, L.ff, ws.hmid, ws.ld_hmid, f32, s);
+  {
+    GemmParams d{ws.hmid, ws.ld_hmid, L.w_dense_down, B, E, L.ff, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(d, s);
+  }
+  sandwich_add(ws.resid, ws.y, nullptr, 1.f, nullptr, 0.f, B, E, L.norm2_b, L.ls2, cfg.eps, nullptr, nullptr, f32, s);
+}
+
 void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
   if (cfg.block == 1) {
     layer_run_postnorm(ri, B, s);
+    return;
+  }
+  if (cfg.block == 2) {
+    layer_run_sandwich(ri, B, s);
     return;
   }
   const RunDesc& r = runs.at(ri);
@@ -286,6 +393,13 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
 
 void StackExecutor::head(int n_logits, bool use_idx, hipStream_t s) {
   if (n_logits <= 0) return;
+  if (cfg.block == 2) {  // an RMS norm with one number as its weight, and a plain factor on the logits
+    scalar_norm_cast(ws.resid, use_idx ? in.logit_idx : nullptr, n_logits, cfg.E, final_w, cfg.eps, ws.lrows, cfg.f32, s);
+    GemmParams g{ws.lrows, cfg.E, head_w, n_logits, cfg.V, cfg.E, in.logits, in.ld_logits, EPI_SCALE, cfg.logit_scale, nullptr,
+                 0.f, cfg.f32};
+    gemm(g, s);
+    return;
+  }
   layer_norm_cast(ws.resid, use_idx ? in.logit_idx : nullptr, n_logits, cfg.E, final_w, final_b, cfg.eps, ws.lrows, cfg.f32,
                   s);
   GemmParams g{ws.lrows, cfg.E, head_w, n_logits, cfg.V, cfg.E, in.logits, in.ld_logits, EPI_SOFTCAP, 0.f, nullptr,

@@ -17,8 +17,11 @@ struct StackConfig {
   float eps = 1e-5f, residual_mult = 1.f, logit_softcap = 0.f;
   int f32 = 0;
   int max_B = 0, max_seqs = 0;
-  int block = 0;            // 0: one norm, mixer and feed-forward in parallel; 1: norms on the sublayers' outputs
+  int block = 0;            // 0: one norm, mixer and feed-forward in parallel; 1: norms on the sublayers' outputs;
+                            // 2: scalar-weight RMS norms before and after both sublayers
   float embed_scale = 1.f;
+  float logit_scale = 1.f;  // block 2: logits = head x * logit_scale
+  int canon_taps = 1;       // block 2: taps of the convolution added to the mixer's input (1: none)
 };
 
 struct LayerDesc {
@@ -66,6 +69,25 @@ struct LayerDesc {
   const float* dt_bias = nullptr;
   const float* a_log = nullptr;
   const float* d_skip = nullptr;
+  // layers with scalar-weight norms around both sublayers: norm_w / norm_b and norm2_w / norm2_b hold the single
+  // weights of the norms before / after the mixer and the feed-forward
+  const float* in_b = nullptr;      // [n_in] biases of the stacked input projection (zero where there is none)
+  const float* o_b = nullptr;       // [E] bias of the attention's output projection, or null
+  const float* ls1 = nullptr;       // [E] per-channel scale of the mixer's result
+  const float* ls2 = nullptr;       // [E] of the feed-forward's
+  const float* canon = nullptr;     // [E][taps]
+  int qk_norm = 0, v_from_k = 0;
+  const float* q_norm = nullptr;
+  const float* k_norm = nullptr;
+  const float* talk = nullptr;      // [heads][heads] mixing of the heads' attention weights, or null
+  // a gated linear attention that reads the same input; the layer's result is left_scale * attention + right_scale * it
+  int r_heads = 0, r_dim = 0, r_vdim = 0, r_rank = 0;
+  float r_tau = 1.f, left_scale = 1.f, right_scale = 1.f;
+  int off_rq = 0, off_rk = 0, off_rv = 0, off_a1 = 0;
+  const void* a2 = nullptr;
+  const float* a2_b = nullptr;
+  const float* gnorm = nullptr;
+  const void* w_o2 = nullptr;       // [E][r_heads * r_vdim]
 };
 
 struct RunDesc {   // one execution of a layer: its own cache
@@ -104,6 +126,9 @@ struct StackWorkspace {
   float* coef = nullptr;   // [max_B][ld_coef] chunked gated scan: per (row, head) {ln a, b, m}
   int ld_coef = 0;
   float* ctot = nullptr;   // [max chunks][ld_coef / 3] the chunks' summed ln a per head
+  float* hn = nullptr;     // [max_B][E] float32: normed rows before the input convolution (block 2)
+  float* y2 = nullptr;     // [max_B][E] float32: the second mixer's projected output (block 2)
+  float* lna = nullptr;    // chunked gated linear attention: the rows' running log decays (= coef)
   MoeGroupWs moe{};        // grouped routed feed-forward (prompt portions, bfloat16); gu == null: unused
   RetChunkWs ret{};        // chunked retention (prompt portions): chunk table, per-chunk states, o before its norm
 };
@@ -145,6 +170,7 @@ class StackExecutor {
   void embed(int B, hipStream_t s);
   void layer_run(int ri, int B, hipStream_t s);
   void layer_run_postnorm(int ri, int B, hipStream_t s);
+  void layer_run_sandwich(int ri, int B, hipStream_t s);
   void head(int n_logits, bool use_idx, hipStream_t s);
   void forward(int B, int n_logits, bool use_idx, hipStream_t s);
 };

@@ -30,6 +30,8 @@ __device__ __forceinline__ void epi_store(const Epi& e, int m, int n, float acc)
     *c = *c + e.mult * (acc + extra);
   } else if (e.mode == EPI_SOFTCAP && e.cap != 0.f) {
     *c = e.cap * tanhf(acc / e.cap);
+  } else if (e.mode == EPI_SCALE) {
+    *c = e.mult * acc;
   } else {
     *c = acc;
   }
@@ -737,8 +739,11 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
   __shared__ float mg[4][2];
   __shared__ float ag[4][16 * DPL];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int b = blockIdx.x / P.H, h = blockIdx.x % P.H;
+  // output "heads": with vheads = G every (query head, value head) pair, else one per query head
+  const int vh = P.vheads > 1 ? P.vheads : 1, NH = P.H * vh;
+  const int b = blockIdx.x / NH, oh = blockIdx.x % NH, h = oh / vh;
   const int g = h / (P.H / P.G);
+  const int vrow = vh > 1 ? (oh % vh - g) * R.bs : 0;  // from the key's row to the same token's row of the value head
   const int split = blockIdx.y;  // long contexts: blockIdx.y-th of nsplit blocks, 64-key groups dealt round robin
   for (int d = threadIdx.x; d < P.D; d += 256) qs[d] = P.proj[(long long)b * P.ld + P.off_q + h * P.D + d];
   const int n = R.q_len[b];
@@ -789,7 +794,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
     l = l * corr + wave_sum(p);
     m = mn;
     ps[wv][lane] = p;
-    rs[wv][lane] = rowidx;  // a key past the end: row 0 with weight 0
+    rs[wv][lane] = valid ? rowidx + vrow : 0;  // a key past the end: row 0 with weight 0
 #pragma unroll
     for (int c = 0; c < DPL; ++c) acc[c] *= corr;
     __builtin_amdgcn_wave_barrier();
@@ -867,9 +872,16 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
       if (dq * DPL + c < P.Dv) w[2 + dq * DPL + c] = acc[c];
     return;
   }
-  T* out = (T*)P.out + (long long)b * P.ld_out + h * P.Dv;
   if (P.sink) L += expf(P.sink[h] - M);
   const float inv = 1.f / L;
+  if (P.out32) {
+    float* out = P.out32 + (long long)b * P.ld_out32 + oh * P.Dv;
+#pragma unroll
+    for (int c = 0; c < DPL; ++c)
+      if (dq * DPL + c < P.Dv) out[dq * DPL + c] = acc[c] * inv;
+    return;
+  }
+  T* out = (T*)P.out + (long long)b * P.ld_out + oh * P.Dv;
 #pragma unroll
   for (int c = 0; c < DPL; ++c)
     if (dq * DPL + c < P.Dv) st(out + dq * DPL + c, acc[c] * inv);
@@ -888,23 +900,29 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnParams P, int 
     const float ms = w[(long long)sidx * (P.Dv + 2)];
     if (ms != -INFINITY) L += w[(long long)sidx * (P.Dv + 2) + 1] * expf(ms - M);  // a split without keys weighs nothing
   }
-  if (P.sink) L += expf(P.sink[item % P.H] - M);
-  T* out = (T*)P.out + (long long)(item / P.H) * P.ld_out + (item % P.H) * P.Dv;
+  const int vh = P.vheads > 1 ? P.vheads : 1, NH = P.H * vh;  // items are (row, output head)
+  if (P.sink) L += expf(P.sink[(item % NH) / vh] - M);
+  T* out = (T*)P.out + (long long)(item / NH) * P.ld_out + (item % NH) * P.Dv;
+  float* out32 = P.out32 ? P.out32 + (long long)(item / NH) * P.ld_out32 + (item % NH) * P.Dv : nullptr;
   for (int d = lane; d < P.Dv; d += 64) {
     float o = 0.f;
     for (int sidx = 0; sidx < nsplit; ++sidx) {
       const float ms = w[(long long)sidx * (P.Dv + 2)];
       if (ms != -INFINITY) o += w[(long long)sidx * (P.Dv + 2) + 2 + d] * expf(ms - M);
     }
-    st(out + d, o / L);
+    if (out32)
+      out32[d] = o / L;
+    else
+      st(out + d, o / L);
   }
 }
 template <typename T>
 static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipStream_t s) {
   const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
   const int vec = P.D % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
-  const int ns = (P.nsplit > 1 && P.split_ws && (long long)R.B * P.H * P.nsplit * (P.Dv + 2) <= P.split_ws_floats) ? P.nsplit : 1;
-  dim3 grid(R.B * P.H, ns);
+  const int NH = P.H * (P.vheads > 1 ? P.vheads : 1);
+  const int ns = (P.nsplit > 1 && P.split_ws && (long long)R.B * NH * P.nsplit * (P.Dv + 2) <= P.split_ws_floats) ? P.nsplit : 1;
+  dim3 grid(R.B * NH, ns);
   const int per = 16 / (int)sizeof(T);  // elements of a 16-byte load
   if (P.Dv <= 64) {
     const int vvec = P.Dv % 4 == 0 && ldv % 4 == 0 && (sizeof(T) == 2 ? 1 : 0) && ((uintptr_t)P.vc & 15) == 0;  // 8-byte pieces (bf16)
@@ -917,7 +935,7 @@ static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipS
     hipLaunchKernelGGL((attention_decode_kernel<T, 16>), grid, dim3(256), 0, s, P, R, vec, vvec, ns);
   }
   if (ns > 1)
-    hipLaunchKernelGGL(attention_merge_kernel<T>, dim3((R.B * P.H + 3) / 4), dim3(256), 0, s, P, R.B * P.H, ns);
+    hipLaunchKernelGGL(attention_merge_kernel<T>, dim3((R.B * NH + 3) / 4), dim3(256), 0, s, P, R.B * NH, ns);
 }
 
 template <typename T, int RQ, int DC>
@@ -981,7 +999,8 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   __shared__ __attribute__((aligned(16))) uint16_t Vl[32 * LDV];
   const int lane = threadIdx.x, q = lane & 31, hf = lane >> 5;
   const int row0 = tiles[2 * blockIdx.x], nrows = tiles[2 * blockIdx.x + 1];
-  const int h = blockIdx.y, g = h / (P.H / P.G);
+  const int vh = P.vheads > 1 ? P.vheads : 1;  // output heads: (query head, value head) pairs with vheads = G
+  const int oh = blockIdx.y, h = oh / vh, g = h / (P.H / P.G), gv = vh > 1 ? oh % vh : g;
   const int* bt = R.block_table + (long long)R.q_seq[row0] * R.max_blocks;
   const int qrow = row0 + min(q, nrows - 1);
   const int qlen = q < nrows ? R.q_len[qrow] : 0;
@@ -1033,7 +1052,7 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
     for (int i = 0; i < VPL; ++i) {  // keys past the end: the last key's row, their weights are zero
       const int c = lane + 64 * i;
       const int key = min(t0 + c / CH, kmax - 1), seg = c % CH;
-      const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
+      const long long rowidx = (long long)(bt[key / R.bs] * P.G + gv) * R.bs + key % R.bs;
       vs_n[i] = *(const u32x4*)(vc + rowidx * ldv + 8 * seg);
     }
   };
@@ -1120,13 +1139,21 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       }
   }
   if (q < nrows) {  // register r of tile j: value dim 32 j + (r & 3) + 8 (r >> 2) + 4 hf of this lane's query
-    bf16* out = (bf16*)P.out + (long long)qrow * P.ld_out + h * DV;
     if (P.sink) li += expf(P.sink[h] - mi);  // the sink: a term of the denominator without key or value
     const float inv = 1.f / li;
+    if (P.out32) {
+      float* out = P.out32 + (long long)qrow * P.ld_out32 + oh * DV;
 #pragma unroll
-    for (int j = 0; j < NV; ++j)
+      for (int j = 0; j < NV; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st(out + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hf, o[j][r] * inv);
+        for (int r = 0; r < 16; ++r) out[32 * j + (r & 3) + 8 * (r >> 2) + 4 * hf] = o[j][r] * inv;
+    } else {
+      bf16* out = (bf16*)P.out + (long long)qrow * P.ld_out + oh * DV;
+#pragma unroll
+      for (int j = 0; j < NV; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st(out + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hf, o[j][r] * inv);
+    }
   }
 }
 // (key size / 16, value size / 32) the kernel is built for: equal key and value sizes 64 / 96 / 128, and the rows of
@@ -1142,8 +1169,10 @@ bool flash_prefill_supported(const AttnParams& P) {
          ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
 }
 void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {
-  check(flash_prefill_supported(P) && tiles && ntiles > 0 && P.G > 0 && P.H % P.G == 0 && P.out, "flash prefill: operands");
-  dim3 grid(ntiles, P.H);
+  check(flash_prefill_supported(P) && tiles && ntiles > 0 && P.G > 0 && P.H % P.G == 0 && (P.out || P.out32) &&
+            (P.vheads <= 1 || P.vheads == P.G),
+        "flash prefill: operands");
+  dim3 grid(ntiles, P.H * (P.vheads > 1 ? P.vheads : 1));
 #define FLASH_LAUNCH(KD, NV)                  \
   if (P.D == 16 * KD && P.Dv == 32 * NV)      \
     hipLaunchKernelGGL((flash_prefill_kernel<KD, NV>), grid, dim3(64), 0, s, P, R, tiles);
@@ -1152,9 +1181,11 @@ void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int
   launched("flash_prefill");
 }
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
-  check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && P.out,
+  check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && (P.out || P.out32) &&
+            (P.vheads <= 1 || P.vheads == P.G),
         "attention: head sizes up to 256, heads a multiple of key/value heads");
-  if (R.B * P.H <= 1024) {  // decode steps (and short portions): a block per (row, head)
+  // decode steps (and short portions): a block per (row, head); so are float32 outputs and (query head, value head) pairs
+  if (R.B * P.H <= 1024 || P.out32 || P.vheads > 1) {
     if (P.f32)
       launch_attention_decode<float>(P, R, s);
     else

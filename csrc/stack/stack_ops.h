@@ -9,12 +9,13 @@
 namespace omx {
 namespace stack {
 
-enum { EPI_STORE = 0, EPI_RESID = 1, EPI_SOFTCAP = 2 };
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_SOFTCAP = 2, EPI_SCALE = 3 };
 
 // C = epi(A . W^T): A [M][K] (row stride lda) and W [N][K] in the matrix dtype, float32 accumulation.
 //   EPI_STORE:   C[m][n] = acc                                    (C float32, row stride ldc)
 //   EPI_RESID:   C[m][n] += mult * (acc + (add ? add[m][n] : 0))  (C = the residual stream; add stride ldc)
 //   EPI_SOFTCAP: C[m][n] = cap ? cap * tanh(acc / cap) : acc
+//   EPI_SCALE:   C[m][n] = mult * acc
 struct GemmParams {
   const void* A;
   int lda;
@@ -73,6 +74,11 @@ struct AttnParams {
   // of a cached row are its value too (latent attention: one row per token serves every head)
   int ldk, ldv;
   const float* sink;    // [H] or null: exp(sink[h]) joins the softmax denominator (no key, no value, not scaled)
+  // vheads = G: every query head meets the values of EVERY key/value head, output "head" h * G + c holds query head
+  // h's weights on the values of key/value head c (what a mixing of the heads' weights needs); 0 or 1: its own only
+  int vheads;
+  float* out32;         // non-null: the outputs leave in float32 here (row stride ld_out32) instead of `out`
+  int ld_out32;
 };
 // q *= 1 + coef * ln(floor((pos + 1) / every) + 1); k, v of every row stored at its slot
 void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);
@@ -275,6 +281,94 @@ void group_rms_cast(const float* y, int ld_y, int rows, int n, int groups, const
                     int ld_gate, void* out, int ld_out, int f32, hipStream_t s);
 // out = relu(z)^2, matrix dtype
 void relu2_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
+
+// ---- layers with scalar-weight RMS norms before and after both sublayers (stack_sandwich.hip)
+// hn[r] = x[r] / rms(x[r]) * g[0] (float32); out[r] = hn[r] + conv(hn)[r] in the matrix dtype, where conv is a causal
+// per-channel convolution over the rows of r's sequence (w [E][taps], the last tap is the current token's) that
+// continues from the sequence's carried window (slot s: window + s * stride = [taps - 1][E], oldest first), which
+// is advanced past the step's rows. taps == 1 (w null): no convolution.
+constexpr int CANON_MAX_TAPS = 8;
+struct CanonParams {
+  const float* x;
+  const float* g;
+  float eps;
+  int E, taps;
+  const float* w;
+  float* window;
+  long long stride;
+  float* hn;            // [B][E]
+  void* out;            // [B][E] matrix dtype
+  int f32;
+};
+void scalar_norm_conv(const CanonParams& P, const StepRows& R, hipStream_t s);
+// out[r] = x[idx ? idx[r] : r] / rms * g[0], matrix dtype
+void scalar_norm_cast(const float* x, const int* idx, int rows, int E, const float* g, float eps, void* out, int f32,
+                      hipStream_t s);
+
+enum { QK_NORM_NONE = 0, QK_NORM_WEIGHT_FIRST = 1, QK_NORM_UNIT_LAST = 2 };
+struct QkPrepParams {
+  float* proj;          // [B][ld] float32: q at off_q (finished in place), k at off_k, v at off_v
+  int ld, off_q, off_k, off_v;
+  const float* bias;    // indexed like proj's columns, or null
+  int H, G, D, Dv;
+  int rot_dims;         // rotate-half pairs (i, i + rot_dims / 2) of every head turn by pos * inv_freq[i]
+  const double* inv_freq;
+  int qk_norm;          // QK_NORM_WEIGHT_FIRST: rms norm * weight before the rotation; QK_NORM_UNIT_LAST: unit rms after
+  const float* q_norm;  // [D]
+  const float* k_norm;
+  float eps;
+  int v_from_k;         // the value row is the key as projected (bias added, before norm and rotation); Dv == D
+  void* kc;             // [blocks][G][bs][D]
+  void* vc;             // [blocks][G][bs][Dv]
+  int f32;
+};
+void qk_prepare(const QkPrepParams& P, const StepRows& R, hipStream_t s);
+// out[b][h] = sum_g talk[h][g] * o32[b][g * G + kv(h)] (vectors of Dv): the mixed weights of head h on the values of
+// its own key/value head, from the attention's outputs of every (query head, value head) pair
+void talk_mix(const float* o32, int ld_o, int B, int H, int G, int Dv, const float* talk, void* out, int ld_out, int f32,
+              hipStream_t s);
+
+// gated linear attention: S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t D^(-1/2)), with
+// alpha = sigmoid(z)^(1 / tau), z = a2 . a1_t + a2_b per key channel; out = rms_norm(o per head) * norm_w * silu(g)
+struct GlaParams {
+  const float* proj;    // [B][ld] float32
+  int ld, off_q, off_k, off_v, off_g, off_a1;
+  int H, D, Dv, rank;
+  const void* a2;       // [H * D][rank] matrix dtype
+  const float* a2_b;    // [H * D]
+  float tau;
+  const float* norm_w;  // [Dv]
+  float eps;
+  float* state;         // slot s: state + s * state_stride = S [H][D][Dv] float32
+  long long state_stride;
+  void* out;            // [B][ld_out] matrix dtype, head-major
+  int ld_out;
+  int f32;
+};
+void gla(const GlaParams& P, const StepRows& R, hipStream_t s);
+bool gla_supported(int D, int Dv);
+// the same in chunks (prompt portions) over the host-built chunk table of the chunked retention; lna [B][H * D] and
+// U / Sin (one state per chunk) are scratch, raw [B][ld_raw] receives o before its norm
+struct GlaChunkWs {
+  const int* chunks;
+  int nchunks, max_chunks;
+  float* U;
+  float* Sin;
+  long long u_stride;
+  float* lna;
+  int ld_lna;
+  float* raw;
+  int ld_raw;
+};
+void gla_chunked(const GlaParams& P, const StepRows& R, const GlaChunkWs& W, hipStream_t s);
+bool gla_chunk_supported(int D, int Dv);
+
+// x[r] += ls * (v / rms(v) * g[0]) with v = sa * (y[r] + bias) + (y2 ? sb * y2[r] : 0); with g_next and hout the
+// updated row also leaves normed, x_new / rms(x_new) * g_next[0], in the matrix dtype (the next sublayer's operand)
+void sandwich_add(float* x, const float* y, const float* bias, float sa, const float* y2, float sb, int rows, int E,
+                  const float* g, const float* ls, float eps, const float* g_next, void* hout, int f32, hipStream_t s);
+// out = gelu_tanh(z[:, :F]) * z[:, F:2F], matrix dtype
+void geglu_tanh_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
 
 }  // namespace stack
 }  // namespace omx

@@ -247,6 +247,8 @@ class StackRunner(Runner):
                                                for s in cfg.layers), **f32)
         # chunked retention of prompt portions: the chunk table and one state per chunk (its U, its incoming state)
         rets = [s.mixer for s in cfg.layers if s.mixer.kind in (MIX_RETENTION, MIX_MLSTM, MIX_MAMBA2)]
+        glas = [s.mixer.right for s in cfg.layers if s.mixer.right is not None]  # gated linear attention beside attention
+        rets += glas
         n_ch = max_batch // 32 + max_seqs + 1 if rets and max_batch > 16 else 1
         self.d_chunks = torch.zeros(n_ch, 4, **i32)
         self.d_tiles = torch.zeros(max_batch // 32 + max_seqs + 1, 2, **i32)  # attention query tiles of a step
@@ -254,7 +256,8 @@ class StackRunner(Runner):
                                  if n_ch > 1 else 1, **f32)
         # chunked gated scans: the rows' {ln decay, input weight, running maximum} per head, the chunks' summed ln decay
         hmax = max([m.heads for m in rets if m.kind != MIX_RETENTION], default=0) if n_ch > 1 else 0
-        self.scan_coef = torch.zeros(max_batch, 3 * hmax, **f32) if hmax else None
+        # (gated linear attention: the rows' running log decays, one per head and key channel)
+        self.scan_coef = torch.zeros(max_batch, max([3 * hmax] + ([m.n_q for m in glas] if n_ch > 1 else [])), **f32) if hmax else None
         self.scan_ctot = torch.zeros(n_ch, hmax, **f32) if hmax else None
         self.ret_sin = torch.zeros_like(self.ret_u)
         # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
