@@ -53,7 +53,7 @@ static void validate_sandwich(const StackExecutor& e, const RunDesc& r, const La
   need(L.qk_norm != QK_NORM_WEIGHT_FIRST || (L.q_norm && L.k_norm), "query / key norm weights missing");
   need(!L.v_from_k || L.vdim == L.dim, "values that are the keys need vdim == dim");
   need(!L.talk || (ws.cbuf && (long long)L.heads * L.kv_heads * L.vdim <= ws.ld_cbuf), "mixed heads: float32 buffer too small");
-  need(taps >= 1 && taps <= CANON_MAX_TAPS && (taps == 1 || (L.canon && r.state)), "input convolution (1..8 taps) operands");
+  need(taps >= 1 && taps <= CANON_MAX_TAPS && L.canon && (taps == 1 || r.state), "input convolution (1..8 taps) operands");
   long long need_state = (long long)(taps - 1) * e.cfg.E;
   int n_out = L.heads * L.vdim;
   if (L.r_heads) {

@@ -21,7 +21,7 @@ struct StackConfig {
                             // 2: scalar-weight RMS norms before and after both sublayers
   float embed_scale = 1.f;
   float logit_scale = 1.f;  // block 2: logits = head x * logit_scale
-  int canon_taps = 1;       // block 2: taps of the convolution added to the mixer's input (1: none)
+  int canon_taps = 1;       // block 2: taps of the convolution added to the mixer's input (1: the current token only)
 };
 
 struct LayerDesc {

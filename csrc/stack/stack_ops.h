@@ -286,7 +286,7 @@ void relu2_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, 
 // hn[r] = x[r] / rms(x[r]) * g[0] (float32); out[r] = hn[r] + conv(hn)[r] in the matrix dtype, where conv is a causal
 // per-channel convolution over the rows of r's sequence (w [E][taps], the last tap is the current token's) that
 // continues from the sequence's carried window (slot s: window + s * stride = [taps - 1][E], oldest first), which
-// is advanced past the step's rows. taps == 1 (w null): no convolution.
+// is advanced past the step's rows. taps == 1: a per-channel factor on the current token, no window.
 constexpr int CANON_MAX_TAPS = 8;
 struct CanonParams {
   const float* x;

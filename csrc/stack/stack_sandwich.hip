@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void scalar_norm_conv_kernel(CanonParams P, St
       const int back = K - 1 - j;
       const float v = back == 0 ? cur : back <= nb ? P.x[(long long)(r - back) * E + c] * scale[back]
                                                    : win[(long long)(K - 1 - (back - nb)) * E + c];
-      if (K > 1) acc += P.w[(long long)c * K + j] * v;
+      acc += P.w[(long long)c * K + j] * v;
       if (alone && back > 0) win[(long long)(K - 1 - back) * E + c] = back == 1 ? cur : win[(long long)(K - back) * E + c];
     }
     st((T*)P.out + (long long)r * E + c, acc);
@@ -69,8 +69,8 @@ __global__ __launch_bounds__(256) void canon_window_kernel(CanonParams P, StepRo
     }
 }
 void scalar_norm_conv(const CanonParams& P, const StepRows& R, hipStream_t s) {
-  check(R.B > 0 && P.x && P.g && P.hn && P.out && P.E > 0 && P.taps >= 1 && P.taps <= CANON_MAX_TAPS &&
-            (P.taps == 1 || (P.w && P.window)),
+  check(R.B > 0 && P.x && P.g && P.hn && P.out && P.E > 0 && P.taps >= 1 && P.taps <= CANON_MAX_TAPS && P.w &&
+            (P.taps == 1 || P.window),
         "scalar_norm_conv: bad operands (at most 8 taps)");
   if (P.f32)
     hipLaunchKernelGGL(scalar_norm_conv_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R);

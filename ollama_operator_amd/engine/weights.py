@@ -564,7 +564,7 @@ class StackWeights:
         E, m, f = cfg.n_embd, spec.mixer, spec.mlp
         L: dict = {k: vec(get(p + k, ())) for k in ("norm1", "norm1b")}
         L["ls1"] = vec(get(p + "ls1", (E,)))
-        L["canon"] = vec(get(p + "canon1", (E, cfg.canon_taps))) if cfg.canon_taps > 1 else None
+        L["canon"] = vec(get(p + "canon1", (E, cfg.canon_taps)))  # one tap: a per-channel factor on the current token
         a = p + ("mix.left." if m.right is not None else "mix.")
         parts, off, bias, n = [], {}, [], 0
 

@@ -422,7 +422,8 @@ class StackConfig:
     block: int = BLOCK_PARALLEL
     embed_scale: float = 1.0
     logit_scale: float = 1.0    # logits = head x * logit_scale
-    canon_taps: int = 1         # sandwich block: taps of the convolution added to the mixer's input (1 = none)
+    canon_taps: int = 1         # sandwich block: taps of the convolution added to the mixer's input (the last one is
+                                # the current token's; with 1 nothing is carried between tokens)
     ctx_len: int = 1 << 20      # the design has no positional table: bounded by the cache pool only
     bos_id: int = 0
     eos_id: int = -1            # no tokenizer ships with these models: generation never stops on a token

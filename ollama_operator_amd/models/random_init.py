@@ -66,6 +66,8 @@ def write_random_stack(path: str, cfg, seed: int = 0, std: float = 0.05) -> None
     from .config import MIX_RETENTION
     if cfg.arch == "norevik":
         return write_random_norevik(path, cfg, seed=seed)
+    if cfg.arch == "suvunex":
+        return write_random_suvunex(path, cfg, seed=seed)
     g = torch.Generator().manual_seed(seed)
     E, V = cfg.n_embd, cfg.n_vocab
     T: dict = {}
@@ -192,4 +194,81 @@ def write_random_norevik(path: str, cfg, seed: int = 0) -> None:
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as fh:
         json.dump(cfg.to_norevik(), fh, indent=1)
+    write_safetensors(os.path.join(path, "model.safetensors"), T)
+
+
+def write_random_suvunex(path: str, cfg, seed: int = 0) -> None:
+    """Random-init model folder of the Suvunex design (its tensor names). Projections ~ N(0, 1 / fan-in) with biases
+    of a fraction of a unit; scalar norm weights and per-channel scales near 1; convolution taps of a fraction of
+    the identity; sinks of a few units; a head-mixing matrix near the identity; decay biases spread so that some
+    key channels forget in a few tokens and others keep for hundreds."""
+    import json
+    import os
+
+    import torch
+
+    from ..engine.safetensors_io import write_safetensors
+    g = torch.Generator().manual_seed(seed)
+    E, V = cfg.n_embd, cfg.n_vocab
+    T: dict = {}
+
+    def rnd(name, shape, s, mean=0.0):
+        T[name] = (mean + s * torch.randn(tuple(shape), generator=g)).to(torch.bfloat16)
+
+    def uni(name, shape, lo, hi):
+        T[name] = (lo + (hi - lo) * torch.rand(tuple(shape), generator=g)).to(torch.bfloat16)
+
+    def lin(name, n_out, n_in, gain=1.0, bias=False):
+        rnd(name, (n_out, n_in), gain / n_in ** 0.5)
+        if bias:
+            rnd(name + ".b", (n_out,), 0.3)
+
+    def attention(a, m):
+        lin(a + "q", m.n_q, E, 1.5, m.bias)
+        lin(a + "k", m.n_k, E, 1.5, m.bias)
+        if not m.v_from_k:
+            lin(a + "v", m.n_v, E, 1.0, m.bias)
+        if m.qk_norm == 1:
+            rnd(a + "q.norm", (m.dim,), 0.2, 1.0)
+            rnd(a + "k.norm", (m.dim,), 0.2, 1.0)
+        if m.sink == 1:
+            uni(a + "sink", (m.heads,), -1.0, 4.0)
+        if m.talk:
+            T[a + "talk"] = (torch.eye(m.heads) + 0.3 * torch.randn(m.heads, m.heads, generator=g)).to(torch.bfloat16)
+        lin(a + "o", E, m.n_out, 1.0, m.o_bias)
+
+    rnd("embed", (V, E), 1.0 / max(cfg.embed_scale, 1e-6))
+    for i, spec in enumerate(cfg.layers):
+        m, f, p = spec.mixer, spec.mlp, f"l{i}."
+        for k in ("norm1", "norm1b"):
+            rnd(p + k, (), 0.1, 1.0)
+        rnd(p + "ls1", (E,), 0.2, 0.8)
+        rnd(p + "canon1", (E, cfg.canon_taps), 0.3)
+        if m.right is not None:
+            r, b = m.right, p + "mix.right."
+            attention(p + "mix.left.", m)
+            rank = r.decay_rank or 8
+            lin(b + "q", r.n_q, E, 1.5)
+            lin(b + "k", r.n_q, E, 1.5)
+            lin(b + "v", r.n_out, E)
+            lin(b + "g", r.n_out, E, 1.5)
+            lin(b + "a1", rank, E)
+            lin(b + "a2", r.n_q, rank, 2.0)
+            uni(b + "a2.b", (r.n_q,), -1.0, 6.0)
+            rnd(b + "norm", (r.vdim,), 0.1, 1.0)
+            lin(b + "o", E, r.n_out)
+        else:
+            attention(p + "mix.", m)
+        if f is not None:
+            for k in ("norm2", "norm2b"):
+                rnd(p + k, (), 0.1, 1.0)
+            rnd(p + "ls2", (E,), 0.2, 0.8)
+            lin(p + "mlp.gate", f.ff, E, 1.5)
+            lin(p + "mlp.up", f.ff, E)
+            lin(p + "mlp.down", E, f.ff)
+    rnd("final.norm", (), 0.1, 1.0)
+    lin("head", V, E)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(cfg.to_suvunex(), fh, indent=1)
     write_safetensors(os.path.join(path, "model.safetensors"), T)

@@ -643,9 +643,13 @@ class TorchStackExecutor:
         st = r.states[ri]
         hn = stack_scalar_norm(x, L["norm1"], eps)
         r.hn[:B] = hn
-        if cfg.canon_taps > 1:
-            nS = st.shape[1] - (cfg.canon_taps - 1) * E
-            hn = stack_canon_conv(hn, L["canon"].view(E, cfg.canon_taps), st[:, nS:].view(st.shape[0], cfg.canon_taps - 1, E), qseq)
+        taps = cfg.canon_taps
+        if taps > 1:
+            nS = st.shape[1] - (taps - 1) * E
+            window = st[:, nS:].view(st.shape[0], taps - 1, E)
+        else:  # one tap: a per-channel factor on the current token, nothing carried
+            window = torch.zeros(r.max_seqs, 0, E, device=hn.device)
+        hn = stack_canon_conv(hn, L["canon"].view(E, taps), window, qseq)
         r.hbuf[:B] = hn.to(T)
         proj = stack_matmul(r.hbuf[:B], L["w_in"])
         r.proj[:B, :proj.shape[1]] = proj

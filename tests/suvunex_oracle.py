@@ -50,6 +50,8 @@ def input_conv(h, w):
 def rotary_frequencies(rot):
     """f_i = base^(-2i / dims), then the scaling the config names: none, all divided by `factor`, or by wavelength
     bands (short waves kept, long waves divided by `factor`, a linear blend in between)."""
+    if not rot or not rot.get("dims"):
+        return torch.zeros(0, dtype=F64)   # no rotation
     dims = rot["dims"]
     f = [rot["base"] ** (-2.0 * i / dims) for i in range(dims // 2)]
     sc = rot.get("scaling")
@@ -89,7 +91,7 @@ def softmax_plus_one_attention(h, W, m, eps):
     q = (h @ W["q"].T + W["q.b"]).view(n, H, D)
     k = (h @ W["k"].T + W["k.b"]).view(n, G, D)
     v = (h @ W["v"].T + W["v.b"]).view(n, G, Dv)
-    fr = rotary_frequencies(m["rot"])
+    fr = rotary_frequencies(m.get("rot"))
     q, k = unit_rms(rotate_half(q, pos, fr), eps), unit_rms(rotate_half(k, pos, fr), eps)
     mask = torch.tril(torch.ones(n, n, dtype=torch.bool))
     out = torch.zeros(n, H, Dv, dtype=F64)
@@ -136,7 +138,7 @@ def talking_attention(h, W, m, eps):
     q = (h @ W["q"].T + W["q.b"]).view(n, H, D)
     k = (h @ W["k"].T + W["k.b"]).view(n, G, D)
     v = k.clone()
-    fr = rotary_frequencies(m["rot"])
+    fr = rotary_frequencies(m.get("rot"))
     q = rotate_half(unit_rms(q, eps) * W["q.norm"], pos, fr)
     k = rotate_half(unit_rms(k, eps) * W["k.norm"], pos, fr)
     mask = torch.tril(torch.ones(n, n, dtype=torch.bool))
