@@ -368,6 +368,37 @@ NOREVIK_SIZES = {
 }
 
 
+# the Suvunex design at the same widths: two pair layers (softmax attention with a zero-score sink beside gated linear
+# attention), a mixed-heads attention whose values are its keys, a pair layer, twice; four-tap input convolutions;
+# dense gated feed-forwards as wide as the routed models' active hidden units (2 experts + the shared one)
+SUVUNEX_SIZES = {
+    "s": dict(E=1024, pattern="ppap" * 2, H=16, G=4, D=64, F=2048, gla=(8, 64, 128), rank=16),
+    "m": dict(E=2048, pattern="ppap" * 2, H=16, G=4, D=128, F=4096, gla=(16, 64, 128), rank=32),
+}
+
+
+def suvunex_config(z: dict, vocab: int = 32000):
+    """A Suvunex model with the sizes of a real model's layers (random weights)."""
+    from ollama_operator_amd.models.config import (BLOCK_SANDWICH, FF_GLU, MIX_ATTENTION, MIX_GLA, QK_NORM_UNIT_LAST,
+                                                    QK_NORM_WEIGHT_FIRST, SINK_LEARNED, SINK_ONE, LayerSpec, MixerSpec, MoESpec,
+                                                    StackConfig)
+    layers = []
+    for c in z["pattern"]:
+        if c == "p":
+            h, d, dv = z["gla"]
+            m = MixerSpec(kind=MIX_ATTENTION, heads=z["H"], kv_heads=z["G"], dim=z["D"], vdim=z["D"], scale=z["D"] ** -0.5,
+                          rot_dims=z["D"] // 2, rot_base=1e4, rot_scaling=("bands", 4.0, 1.0, 2.0, 4096.0), bias=True, o_bias=True,
+                          qk_norm=QK_NORM_UNIT_LAST, sink=SINK_ONE, left_scale=0.7, right_scale=1.3,
+                          right=MixerSpec(kind=MIX_GLA, heads=h, kv_heads=h, dim=d, vdim=dv, tau=8.0, decay_rank=z["rank"]))
+        else:
+            m = MixerSpec(kind=MIX_ATTENTION, heads=z["H"], kv_heads=z["G"], dim=z["D"], vdim=z["D"], scale=z["D"] ** -0.5,
+                          rot_dims=z["D"], rot_base=1e6, rot_scaling=("linear", 2.0), bias=True, qk_norm=QK_NORM_WEIGHT_FIRST,
+                          sink=SINK_LEARNED, talk=True, v_from_k=True)
+        layers.append(LayerSpec(mixer=m, mlp=MoESpec(kind=FF_GLU, ff=z["F"])))
+    return StackConfig(arch="suvunex", n_vocab=vocab, n_embd=z["E"], layers=layers, norm_eps=1e-6, block=BLOCK_SANDWICH,
+                       embed_scale=float(z["E"]) ** 0.5, canon_taps=4, logit_scale=0.5)
+
+
 def norevik_config(z: dict, vocab: int = 32000):
     """A Norevik model with the sizes of a real model's layers (random weights)."""
     from ollama_operator_amd.models.config import (BLOCK_POSTNORM, FF_DENSE, FF_MOE, MIX_LATENT, MIX_MAMBA2, MIX_MLSTM,
@@ -454,10 +485,12 @@ def bench_stack(a) -> None:
         d = os.path.join(a.dir, f"bizulix-{name}")
         if not os.path.exists(os.path.join(d, "model.safetensors")):
             write_random_stack(d, stack_config(z), seed=0, std=0.02)
-        r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
-        r.warmup()
-        out[name] = {"bizulix_bf16": measure(r), "weights_gb": round(r.w.nbytes / 1e9, 3)}
-        r.close()
+        out[name] = {}
+        if not a.no_bizulix:
+            r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+            r.warmup()
+            out[name] = {"bizulix_bf16": measure(r), "weights_gb": round(r.w.nbytes / 1e9, 3)}
+            r.close()
         if a.norevik:  # the Norevik design at the same width and depth, through the same engine and measurement
             d = os.path.join(a.dir, f"norevik-{name}")
             if not os.path.exists(os.path.join(d, "model.safetensors")):
@@ -466,6 +499,15 @@ def bench_stack(a) -> None:
             r.warmup()
             out[name]["norevik_bf16"] = measure(r)
             out[name]["norevik_weights_gb"] = round(r.w.nbytes / 1e9, 3)
+            r.close()
+        if a.suvunex:  # the Suvunex design at the same width and depth, through the same engine and measurement
+            d = os.path.join(a.dir, f"suvunex-{name}")
+            if not os.path.exists(os.path.join(d, "model.safetensors")):
+                write_random_stack(d, suvunex_config(SUVUNEX_SIZES[name]), seed=0)
+            r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+            r.warmup()
+            out[name]["suvunex_bf16"] = measure(r)
+            out[name]["suvunex_weights_gb"] = round(r.w.nbytes / 1e9, 3)
             r.close()
         if not a.stack_only:
             cfg = ModelConfig(name=f"mixtral-like-{name}", n_vocab=32000, n_embd=z["E"], n_layer=len(z["pattern"]),
@@ -491,6 +533,9 @@ def main():
     ap.add_argument("--stack-only", action="store_true", help="with --stack: skip the comparison model")
     ap.add_argument("--norevik", action="store_true", help="with --stack: also measure the Norevik design (latent "
                     "attention, mLSTM, Mamba-2, score-routed experts) at the same widths")
+    ap.add_argument("--no-bizulix", action="store_true", help="with --stack: skip the Bizulix model (profiles of one design)")
+    ap.add_argument("--suvunex", action="store_true", help="with --stack: also measure the Suvunex design (attention with "
+                    "sinks beside gated linear attention, mixed-heads attention, input convolutions) at the same widths")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--tp", type=int, default=1, help="tensor-parallel degree: one sequence sharded over T GPUs")
     ap.add_argument("--allow-shared", action="store_true",

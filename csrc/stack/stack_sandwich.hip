@@ -32,24 +32,30 @@ __global__ __launch_bounds__(256) void scalar_norm_conv_kernel(CanonParams P, St
   while (nb < K - 1 && r - nb - 1 >= 0 && R.q_seq[r - nb - 1] == seq) ++nb;
   const bool alone = nb == 0 && !(r + 1 < R.B && R.q_seq[r + 1] == seq);
   const float g = P.g[0];
-  float scale[CANON_MAX_TAPS];
-  for (int k = 0; k <= nb; ++k) {
-    const float* xr = P.x + (long long)(r - k) * E;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < E; c += 256) ss += xr[c] * xr[c];
-    scale[k] = g / sqrtf(block_sum256(ss, red) / (float)E + P.eps);
+  float scale[CANON_MAX_TAPS];  // indexed by constants only (unrolled), so it lives in registers
+#pragma unroll
+  for (int k = 0; k < CANON_MAX_TAPS; ++k) {
+    scale[k] = 0.f;
+    if (k <= nb) {  // uniform over the block
+      const float* xr = P.x + (long long)(r - k) * E;
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < E; c += 256) ss += xr[c] * xr[c];
+      scale[k] = g / sqrtf(block_sum256(ss, red) / (float)E + P.eps);
+    }
   }
   float* win = P.window ? P.window + (long long)seq * P.stride : nullptr;
   for (int c = threadIdx.x; c < E; c += 256) {
     const float cur = P.x[(long long)r * E + c] * scale[0];
     P.hn[(long long)r * E + c] = cur;
     float acc = cur;
-    for (int j = 0; j < K; ++j) {
-      const int back = K - 1 - j;
-      const float v = back == 0 ? cur : back <= nb ? P.x[(long long)(r - back) * E + c] * scale[back]
-                                                   : win[(long long)(K - 1 - (back - nb)) * E + c];
-      acc += P.w[(long long)c * K + j] * v;
-      if (alone && back > 0) win[(long long)(K - 1 - back) * E + c] = back == 1 ? cur : win[(long long)(K - back) * E + c];
+#pragma unroll
+    for (int back = CANON_MAX_TAPS - 1; back >= 0; --back) {  // oldest input first, as the taps are stored
+      if (back < K) {
+        const float v = back == 0 ? cur : back <= nb ? P.x[(long long)(r - back) * E + c] * scale[back]
+                                                     : win[(long long)(K - 1 - (back - nb)) * E + c];
+        acc += P.w[(long long)c * K + (K - 1 - back)] * v;
+        if (alone && back > 0) win[(long long)(K - 1 - back) * E + c] = back == 1 ? cur : win[(long long)(K - back) * E + c];
+      }
     }
     st((T*)P.out + (long long)r * E + c, acc);
   }
@@ -119,9 +125,12 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(QkPrepParams P, StepRow
   float* row = P.proj + (long long)b * P.ld;
   const int pos = R.pos[b], half = P.rot_dims / 2, D = P.D;
   for (int i = threadIdx.x; i < half; i += 256) {
+    // the angle and its reduction to [-pi, pi] in float64 (a float32 angle at position 10^3 is off by 10^-4); the
+    // sine and cosine of the reduced angle in float32
     const double ang = (double)pos * P.inv_freq[i];
-    cs[i] = (float)cos(ang);
-    sn[i] = (float)sin(ang);
+    const float red = (float)(ang - 6.283185307179586 * rint(ang * 0.15915494309189535));
+    cs[i] = cosf(red);
+    sn[i] = sinf(red);
   }
   const int slot = R.slot[b];
   const long long blk = slot / R.bs, off = slot % R.bs;
@@ -221,7 +230,7 @@ __global__ __launch_bounds__(256) void talk_mix_kernel(const float* __restrict__
   const long long b = blockIdx.x;
   const float* src = o32 + b * ld_o;
   const int per = H / G;
-  for (int i = threadIdx.x; i < H * Dv; i += 256) {
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < H * Dv; i += 256 * gridDim.y) {
     const int h = i / Dv, d = i % Dv, c = h / per;
     float acc = 0.f;
     for (int g = 0; g < H; ++g) acc += talk[h * H + g] * src[(long long)(g * G + c) * Dv + d];
@@ -233,9 +242,11 @@ void talk_mix(const float* o32, int ld_o, int B, int H, int G, int Dv, const flo
   check(B > 0 && o32 && talk && out && H > 0 && G > 0 && H % G == 0 && ld_o >= H * G * Dv && ld_out >= H * Dv,
         "talk_mix: bad operands");
   if (f32)
-    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(B), dim3(256), 0, s, o32, ld_o, H, G, Dv, talk, (float*)out, ld_out);
+    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(B, (H * Dv + 255) / 256), dim3(256), 0, s, o32, ld_o, H, G, Dv, talk,
+                       (float*)out, ld_out);
   else
-    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(B), dim3(256), 0, s, o32, ld_o, H, G, Dv, talk, (bf16*)out, ld_out);
+    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(B, (H * Dv + 255) / 256), dim3(256), 0, s, o32, ld_o, H, G, Dv, talk,
+                       (bf16*)out, ld_out);
   launched("talk_mix");
 }
 
@@ -354,8 +365,8 @@ void gla(const GlaParams& P, const StepRows& R, hipStream_t s) {
 //   3. gla_out_kernel: every chunk's outputs from its incoming state, in parallel, with the norm and the gate
 constexpr int GC = 32;
 constexpr int GLA_CD = 128;  // largest key size of the chunked form
-// LDS floats of the output kernel: q, k and the running log decays [GC][D + 1] each, A [GC][GC + 1], v [GC][Dv], partials
-static inline long long gla_out_lds(int D, int Dv) { return 3LL * GC * (D + 1) + GC * (GC + 1) + (long long)GC * Dv + 260; }
+// LDS floats of the output kernel: q, k and the running log decays [GC][D + 1] each, A [GC][GC + 1], v [GC][Dv]
+static inline long long gla_out_lds(int D, int Dv) { return 3LL * GC * (D + 1) + GC * (GC + 1) + (long long)GC * Dv; }
 bool gla_chunk_supported(int D, int Dv) {
   return D > 0 && D <= GLA_CD && Dv > 0 && Dv <= 256 && gla_out_lds(D, Dv) * 4 <= 64 * 1024;
 }
@@ -421,8 +432,7 @@ __global__ __launch_bounds__(256) void gla_chunk_scan_kernel(GlaParams P, const 
   }
   st0[e] = S;
 }
-// outputs of one chunk and head: thread t < n first builds its row of A in LDS (the exponentials are per pair and
-// channel), then thread (g, j) sums S^T (q exp(L)) over its rows i and every thread j < Dv finishes row by row
+// outputs of one chunk and head: A is built in LDS first (the exponentials are per pair and channel)
 template <typename T>
 __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __restrict__ chunks, const float* __restrict__ lna,
                                                       int ld_lna, const float* __restrict__ Sin, long long u_stride) {
@@ -435,8 +445,6 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
   float* Lc = kk + GC * D1;        // [GC][D + 1]
   float* A = Lc + GC * D1;         // [GC][GC + 1]
   float* vs = A + GC * (GC + 1);   // [GC][Dv]
-  float* po = vs + GC * Dv;        // [256]
-  float* red = po + 256;           // [4]
   const float qscale = 1.f / sqrtf((float)D);
   for (int i = tid; i < n * D; i += 256) {
     const int t = i / D, d = i % D;
@@ -460,27 +468,50 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
     qd[t * D1 + d] *= expf(Lc[t * D1 + d]);
   }
   __syncthreads();
+  // O = (Q * exp(L)) S + A V: thread (g, j) owns column j of rows t = g, g + NG, ... (up to GC / NG of them) and sums
+  // them whole, the state's column read once per key channel; the rows then meet in LDS for their norms
   const int g = tid / Dv, j = tid % Dv;
-  const bool act = g < NG;
   const float* S = Sin + (long long)c * u_stride + (long long)h * D * Dv;
-  for (int t = 0; t < n; ++t) {
-    float part = 0.f;
-    if (act) {
-      for (int i = g; i < D; i += NG) part += S[(long long)i * Dv + j] * qd[t * D1 + i];
-      for (int sidx = g; sidx <= t; sidx += NG) part += A[t * (GC + 1) + sidx] * vs[sidx * Dv + j];
+  float acc[GC];
+#pragma unroll
+  for (int k = 0; k < GC; ++k) acc[k] = 0.f;
+  if (g < NG) {
+    for (int i = 0; i < D; ++i) {
+      const float sv = S[(long long)i * Dv + j];
+#pragma unroll
+      for (int k = 0; k < GC; ++k) {
+        const int t = g + k * NG;
+        if (t < n) acc[k] += sv * qd[t * D1 + i];
+      }
     }
-    po[tid] = part;
-    __syncthreads();
-    float o = 0.f;
-    if (tid < Dv)
-      for (int gg = 0; gg < NG; ++gg) o += po[gg * Dv + tid];
-    const float ms = block_sum256(o * o, red) / (float)Dv;
-    if (tid < Dv) {
-      const float y = o / sqrtf(ms + P.eps) * P.norm_w[tid] *
-                      silu(P.proj[(long long)(r0 + t) * P.ld + P.off_g + h * Dv + tid]);
-      st((T*)P.out + (long long)(r0 + t) * P.ld_out + h * Dv + tid, y);
+    for (int sidx = 0; sidx < n; ++sidx) {
+      const float vv = vs[sidx * Dv + j];
+#pragma unroll
+      for (int k = 0; k < GC; ++k) {
+        const int t = g + k * NG;
+        if (t < n && sidx <= t) acc[k] += A[t * (GC + 1) + sidx] * vv;
+      }
     }
-    __syncthreads();
+  }
+  __syncthreads();  // every thread is done with vs: the rows' outputs take its place
+  float* ob = vs;   // [GC][Dv]
+  if (g < NG) {
+#pragma unroll
+    for (int k = 0; k < GC; ++k) {
+      const int t = g + k * NG;
+      if (t < n) ob[t * Dv + j] = acc[k];
+    }
+  }
+  __syncthreads();
+  const int lane = tid & 63, wv = tid >> 6;
+  for (int t = wv; t < n; t += 4) {  // a wave per row: the head's RMS norm, its weight, the gate
+    float ss = 0.f;
+    for (int d = lane; d < Dv; d += 64) ss += ob[t * Dv + d] * ob[t * Dv + d];
+    const float inv = 1.f / sqrtf(wave_sum(ss) / (float)Dv + P.eps);
+    for (int d = lane; d < Dv; d += 64) {
+      const float y = ob[t * Dv + d] * inv * P.norm_w[d] * silu(P.proj[(long long)(r0 + t) * P.ld + P.off_g + h * Dv + d]);
+      st((T*)P.out + (long long)(r0 + t) * P.ld_out + h * Dv + d, y);
+    }
   }
 }
 void gla_chunked(const GlaParams& P, const StepRows& R, const GlaChunkWs& W, hipStream_t s) {
@@ -538,9 +569,62 @@ __global__ __launch_bounds__(256) void sandwich_add_kernel(float* __restrict__ x
   const float sn = g_next[0] / sqrtf(block_sum256(s2, red) / (float)E + eps);
   for (int i = threadIdx.x; i < E; i += 256) st(hout + r * E + i, xr[i] * sn);
 }
+// the same with the row held in registers (widths up to 256 * SW_REG): x, y and y2 are read once
+constexpr int SW_REG = 16;
+template <typename T>
+__global__ __launch_bounds__(256) void sandwich_add_reg_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                               const float* __restrict__ bias, float sa,
+                                                               const float* __restrict__ y2, float sb, int E,
+                                                               const float* __restrict__ g, const float* __restrict__ ls,
+                                                               float eps, const float* __restrict__ g_next, T* __restrict__ hout) {
+  __shared__ float red[4];
+  const long long r = blockIdx.x;
+  float* xr = x + r * E;
+  const float* yr = y + r * E;
+  const float* zr = y2 ? y2 + r * E : nullptr;
+  float v[SW_REG], xv[SW_REG], lv[SW_REG];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < SW_REG; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    v[k] = xv[k] = lv[k] = 0.f;
+    if (i < E) {
+      v[k] = sa * (yr[i] + (bias ? bias[i] : 0.f)) + (zr ? sb * zr[i] : 0.f);
+      xv[k] = xr[i];
+      lv[k] = ls[i];
+    }
+    ss += v[k] * v[k];
+  }
+  const float scale = g[0] / sqrtf(block_sum256(ss, red) / (float)E + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < SW_REG; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    xv[k] = xv[k] + lv[k] * (v[k] * scale);
+    if (i < E) xr[i] = xv[k];
+    s2 += xv[k] * xv[k];
+  }
+  if (!hout) return;
+  const float sn = g_next[0] / sqrtf(block_sum256(s2, red) / (float)E + eps);
+#pragma unroll
+  for (int k = 0; k < SW_REG; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    if (i < E) st(hout + r * E + i, xv[k] * sn);
+  }
+}
 void sandwich_add(float* x, const float* y, const float* bias, float sa, const float* y2, float sb, int rows, int E,
                   const float* g, const float* ls, float eps, const float* g_next, void* hout, int f32, hipStream_t s) {
   check(rows > 0 && E > 0 && x && y && g && ls && (!hout || g_next), "sandwich_add: bad operands");
+  if (E <= 256 * SW_REG) {
+    if (f32)
+      hipLaunchKernelGGL(sandwich_add_reg_kernel<float>, dim3(rows), dim3(256), 0, s, x, y, bias, sa, y2, sb, E, g, ls, eps,
+                         g_next, (float*)hout);
+    else
+      hipLaunchKernelGGL(sandwich_add_reg_kernel<bf16>, dim3(rows), dim3(256), 0, s, x, y, bias, sa, y2, sb, E, g, ls, eps,
+                         g_next, (bf16*)hout);
+    launched("sandwich_add");
+    return;
+  }
   if (f32)
     hipLaunchKernelGGL(sandwich_add_kernel<float>, dim3(rows), dim3(256), 0, s, x, y, bias, sa, y2, sb, E, g, ls, eps, g_next,
                        (float*)hout);
