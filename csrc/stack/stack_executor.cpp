@@ -285,14 +285,11 @@ void StackExecutor::layer_run_sandwich(int ri, int B, hipStream_t s) {
       attention(A, R, s);
     if (L.talk) talk_mix(ws.cbuf, ws.ld_cbuf, B, L.heads, L.kv_heads, L.vdim, L.talk, ws.a, ws.ld_a, f32, s);
   }
-  {
-    GemmParams o{ws.a, ws.ld_a, L.w_o, B, E, n1, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
-    gemm(o, s);
-  }
+  const size_t esz = f32 ? 4 : 2;
+  void* a2 = (char*)ws.a + (size_t)n1 * esz;  // the second mixer's outputs sit beside the attention's
   if (L.r_heads) {
-    const size_t esz = f32 ? 4 : 2;
     GlaParams G{ws.proj, ws.ld_proj, L.off_rq, L.off_rk, L.off_rv, L.off_g, L.off_a1, L.r_heads, L.r_dim, L.r_vdim, L.r_rank, L.a2,
-                L.a2_b, L.r_tau, L.gnorm, cfg.eps, r.state, r.state_stride, (char*)ws.a + (size_t)n1 * esz, ws.ld_a, f32};
+                L.a2_b, L.r_tau, L.gnorm, cfg.eps, r.state, r.state_stride, a2, ws.ld_a, f32};
     if (B > SMALL_B && n_chunks > 0 && ws.ret.U && ws.ret.Sin && ws.lna && ws.ld_coef >= L.r_heads * L.r_dim &&
         ws.ret.u_stride >= gla_floats && gla_chunk_supported(L.r_dim, L.r_vdim)) {
       GlaChunkWs W{ws.ret.chunks, n_chunks, ws.ret.max_chunks, ws.ret.U, ws.ret.Sin, ws.ret.u_stride, ws.lna, ws.ld_coef, nullptr, 0};
@@ -300,13 +297,23 @@ void StackExecutor::layer_run_sandwich(int ri, int B, hipStream_t s) {
     } else {
       gla(G, R, s);
     }
-    GemmParams o{(char*)ws.a + (size_t)n1 * esz, ws.ld_a, L.w_o2, B, E, n2, ws.y2, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
-    gemm(o, s);
   }
   const bool has_ff = L.ff_dense != 0;
-  // the updated rows leave normed for the feed-forward in the same launch
-  sandwich_add(ws.resid, ws.y, L.o_b, L.r_heads ? L.left_scale : 1.f, L.r_heads ? ws.y2 : nullptr, L.right_scale, B, E, L.norm_b,
-               L.ls1, cfg.eps, has_ff ? L.norm2_w : nullptr, has_ff ? ws.h : nullptr, f32, s);
+  const float* g_next = has_ff ? L.norm2_w : nullptr;
+  void* h_next = has_ff ? ws.h : nullptr;  // the updated rows leave normed for the feed-forward in the same launch
+  if (L.r_heads && B <= 8) {  // decode steps: both output projections, their scales and the bias in one launch
+    gemv_pair(ws.a, ws.ld_a, L.w_o, n1, L.o_b, L.left_scale, a2, ws.ld_a, L.w_o2, n2, L.right_scale, B, E, ws.y, E, f32, s);
+    sandwich_add(ws.resid, ws.y, nullptr, 1.f, nullptr, 0.f, B, E, L.norm_b, L.ls1, cfg.eps, g_next, h_next, f32, s);
+  } else {
+    GemmParams o{ws.a, ws.ld_a, L.w_o, B, E, n1, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(o, s);
+    if (L.r_heads) {
+      GemmParams o2{a2, ws.ld_a, L.w_o2, B, E, n2, ws.y2, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+      gemm(o2, s);
+    }
+    sandwich_add(ws.resid, ws.y, L.o_b, L.r_heads ? L.left_scale : 1.f, L.r_heads ? ws.y2 : nullptr, L.right_scale, B, E, L.norm_b,
+                 L.ls1, cfg.eps, g_next, h_next, f32, s);
+  }
   if (!has_ff) return;
   {
     GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};

@@ -367,6 +367,9 @@ bool gla_chunk_supported(int D, int Dv);
 // updated row also leaves normed, x_new / rms(x_new) * g_next[0], in the matrix dtype (the next sublayer's operand)
 void sandwich_add(float* x, const float* y, const float* bias, float sa, const float* y2, float sb, int rows, int E,
                   const float* g, const float* ls, float eps, const float* g_next, void* hout, int f32, hipStream_t s);
+// C[m][n] = sa * (A1[m] . W1[n] + bias[n]) + sb * (A2[m] . W2[n]): two output projections of a few rows (M <= 8) in one launch
+void gemv_pair(const void* A1, int lda1, const void* W1, int K1, const float* bias, float sa, const void* A2, int lda2,
+               const void* W2, int K2, float sb, int M, int N, float* C, int ldc, int f32, hipStream_t s);
 // out = gelu_tanh(z[:, :F]) * z[:, F:2F], matrix dtype
 void geglu_tanh_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
 

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void scalar_norm_conv_kernel(CanonParams P, St
     }
   }
   float* win = P.window ? P.window + (long long)seq * P.stride : nullptr;
-  for (int c = threadIdx.x; c < E; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < E; c += 256 * gridDim.y) {
     const float cur = P.x[(long long)r * E + c] * scale[0];
     P.hn[(long long)r * E + c] = cur;
     float acc = cur;
@@ -78,10 +78,12 @@ void scalar_norm_conv(const CanonParams& P, const StepRows& R, hipStream_t s) {
   check(R.B > 0 && P.x && P.g && P.hn && P.out && P.E > 0 && P.taps >= 1 && P.taps <= CANON_MAX_TAPS && P.w &&
             (P.taps == 1 || P.window),
         "scalar_norm_conv: bad operands (at most 8 taps)");
+  // few rows (decode steps): the channels are shared among several blocks per row (each sums the whole row itself)
+  const dim3 grid(R.B, R.B <= 64 ? std::min(8, (P.E + 255) / 256) : 1);
   if (P.f32)
-    hipLaunchKernelGGL(scalar_norm_conv_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL(scalar_norm_conv_kernel<float>, grid, dim3(256), 0, s, P, R);
   else
-    hipLaunchKernelGGL(scalar_norm_conv_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL(scalar_norm_conv_kernel<bf16>, grid, dim3(256), 0, s, P, R);
   launched("scalar_norm_conv");
   if (P.taps > 1 && R.B > 1) {  // a single row is alone in its sequence
     hipLaunchKernelGGL(canon_window_kernel, dim3(R.B, (P.E + 1023) / 1024), dim3(256), 0, s, P, R);
@@ -137,7 +139,9 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(QkPrepParams P, StepRow
   T* kc = (T*)P.kc;
   T* vc = (T*)P.vc;
   const int heads = P.H + P.G;
-  for (int h0 = 0; h0 < heads; h0 += 4) {  // the same number of turns for every wave: block-wide barriers inside
+  // turns of four heads (a head per wave); with several blocks per row (gridDim.y) a block takes every gridDim.y-th
+  // turn, and every wave of a block sees the same number of turns: block-wide barriers inside
+  for (int h0 = 4 * blockIdx.y; h0 < heads; h0 += 4 * gridDim.y) {
     const int head = h0 + wv;
     const bool on = head < heads, isq = head < P.H;
     const int hh = isq ? head : head - P.H;
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(QkPrepParams P, StepRow
       }
     }
   }
-  if (!P.v_from_k) {
+  if (!P.v_from_k && blockIdx.y == gridDim.y - 1) {
     for (int i = threadIdx.x; i < P.G * P.Dv; i += 256) {
       const int g = i / P.Dv, d = i % P.Dv;
       st(vc + ((blk * P.G + g) * R.bs + off) * P.Dv + d, row[P.off_v + i] + (P.bias ? P.bias[P.off_v + i] : 0.f));
@@ -216,10 +220,13 @@ void qk_prepare(const QkPrepParams& P, const StepRows& R, hipStream_t s) {
             P.rot_dims % 2 == 0 && P.rot_dims <= P.D && (P.rot_dims == 0 || P.inv_freq) &&
             (P.qk_norm != QK_NORM_WEIGHT_FIRST || (P.q_norm && P.k_norm)) && (!P.v_from_k || P.Dv == P.D),
         "qk_prepare: bad operands (head size up to 256)");
+  // few rows (decode steps): a block per turn of four heads, so a row's heads are finished side by side
+  const int turns = (P.H + P.G + 3) / 4;
+  const dim3 grid(R.B, R.B <= 64 ? turns : 1);
   if (P.f32)
-    hipLaunchKernelGGL(qk_prepare_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL(qk_prepare_kernel<float>, grid, dim3(256), 0, s, P, R);
   else
-    hipLaunchKernelGGL(qk_prepare_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL(qk_prepare_kernel<bf16>, grid, dim3(256), 0, s, P, R);
   launched("qk_prepare");
 }
 
@@ -258,15 +265,48 @@ void talk_mix(const float* o32, int ld_o, int B, int H, int G, int Dv, const flo
 // registers; o is a sum of NG partials per column; the head's RMS norm, its weight and the silu gate finish the row.
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 template <typename T>
-__device__ __forceinline__ float gla_ln_alpha(const GlaParams& P, const float* row, int ch) {
+__device__ __forceinline__ void load8w(const T* p, float* out);
+template <>
+__device__ __forceinline__ void load8w<bf16>(const bf16* p, float* out) {
+  const u32x4 a = *(const u32x4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __uint_as_float(a[i] << 16);
+    out[2 * i + 1] = __uint_as_float(a[i] & 0xffff0000u);
+  }
+}
+template <>
+__device__ __forceinline__ void load8w<float>(const float* p, float* out) {
+  const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[i] = a[i];
+    out[4 + i] = b[i];
+  }
+}
+// a1: the row's first decay factor (rank floats, global or LDS); vec: a2's rows allow 16-byte loads (rank % 8 == 0)
+template <typename T>
+__device__ __forceinline__ float gla_ln_alpha(const GlaParams& P, const float* a1, int ch, int vec) {
   const T* w = (const T*)P.a2 + (long long)ch * P.rank;
   float z = P.a2_b[ch];
-  for (int i = 0; i < P.rank; ++i) z += ld(w + i) * row[P.off_a1 + i];
+  if (vec) {
+    for (int i = 0; i < P.rank; i += 8) {
+      float w8[8];
+      load8w<T>(w + i, w8);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) z += w8[u] * a1[i + u];
+    }
+  } else {
+    for (int i = 0; i < P.rank; ++i) z += ld(w + i) * a1[i];
+  }
   return log_sigmoid(z) / P.tau;
 }
+static inline int gla_vec(const GlaParams& P) { return P.rank % 8 == 0 && ((uintptr_t)P.a2 & 15) == 0; }
+constexpr int GLA_MAX_RANK = 256;
 template <typename T, int MAXI>
-__global__ __launch_bounds__(256) void gla_kernel(GlaParams P, StepRows R) {
+__global__ __launch_bounds__(256) void gla_kernel(GlaParams P, StepRows R, int vec) {
   __shared__ float qs[256], ks[256], as[256], vs[256], po[256], red[4];
+  __shared__ float a1s[GLA_MAX_RANK];
   const int r0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int seq = R.q_seq[r0];
   if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;  // not the first row of its segment (uniform per block)
@@ -284,12 +324,14 @@ __global__ __launch_bounds__(256) void gla_kernel(GlaParams P, StepRows R) {
   const float qscale = 1.f / sqrtf((float)D);
   for (int r = r0; r < R.B && R.q_seq[r] == seq; ++r) {
     const float* row = P.proj + (long long)r * P.ld;
+    if (tid < P.rank) a1s[tid] = row[P.off_a1 + tid];
     if (tid < D) {
       qs[tid] = row[P.off_q + h * D + tid] * qscale;
       ks[tid] = row[P.off_k + h * D + tid];
-      as[tid] = expf(gla_ln_alpha<T>(P, row, h * D + tid));
     }
     if (tid < Dv) vs[tid] = row[P.off_v + h * Dv + tid];
+    __syncthreads();
+    if (tid < D) as[tid] = expf(gla_ln_alpha<T>(P, a1s, h * D + tid, vec));
     __syncthreads();
     float part = 0.f;
     if (act) {
@@ -331,16 +373,16 @@ static void launch_gla(const GlaParams& P, const StepRows& R, hipStream_t s) {
   const int ng = 256 / P.Dv, ni = (P.D + ng - 1) / ng;
   const dim3 grid(R.B, P.H);
   if (ni <= 8)
-    hipLaunchKernelGGL((gla_kernel<T, 8>), grid, dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL((gla_kernel<T, 8>), grid, dim3(256), 0, s, P, R, gla_vec(P));
   else if (ni <= 16)
-    hipLaunchKernelGGL((gla_kernel<T, 16>), grid, dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL((gla_kernel<T, 16>), grid, dim3(256), 0, s, P, R, gla_vec(P));
   else if (ni <= 32)
-    hipLaunchKernelGGL((gla_kernel<T, 32>), grid, dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL((gla_kernel<T, 32>), grid, dim3(256), 0, s, P, R, gla_vec(P));
   else
-    hipLaunchKernelGGL((gla_kernel<T, 64>), grid, dim3(256), 0, s, P, R);
+    hipLaunchKernelGGL((gla_kernel<T, 64>), grid, dim3(256), 0, s, P, R, gla_vec(P));
 }
 static void check_gla(const GlaParams& P, const StepRows& R) {
-  check(R.B > 0 && P.proj && P.state && P.out && P.a2 && P.a2_b && P.norm_w && P.H > 0 && P.rank > 0 && P.tau > 0.f &&
+  check(R.B > 0 && P.proj && P.state && P.out && P.a2 && P.a2_b && P.norm_w && P.H > 0 && P.rank > 0 && P.rank <= GLA_MAX_RANK && P.tau > 0.f &&
             gla_supported(P.D, P.Dv),
         "gated linear attention: operands or head sizes (key and value size <= 256, state within the registers)");
 }
@@ -371,10 +413,13 @@ bool gla_chunk_supported(int D, int Dv) {
   return D > 0 && D <= GLA_CD && Dv > 0 && Dv <= 256 && gla_out_lds(D, Dv) * 4 <= 64 * 1024;
 }
 template <typename T>
-__global__ __launch_bounds__(256) void gla_lna_kernel(GlaParams P, int B, float* __restrict__ lna, int ld_lna) {
+__global__ __launch_bounds__(256) void gla_lna_kernel(GlaParams P, int B, float* __restrict__ lna, int ld_lna, int vec) {
+  __shared__ float a1s[GLA_MAX_RANK];
   const int r = blockIdx.x;
   const float* row = P.proj + (long long)r * P.ld;
-  for (int ch = threadIdx.x; ch < P.H * P.D; ch += 256) lna[(long long)r * ld_lna + ch] = gla_ln_alpha<T>(P, row, ch);
+  if (threadIdx.x < P.rank) a1s[threadIdx.x] = row[P.off_a1 + threadIdx.x];
+  __syncthreads();
+  for (int ch = threadIdx.x; ch < P.H * P.D; ch += 256) lna[(long long)r * ld_lna + ch] = gla_ln_alpha<T>(P, a1s, ch, vec);
 }
 __global__ __launch_bounds__(256) void gla_cum_kernel(const int* __restrict__ chunks, int HD, float* __restrict__ lna,
                                                       int ld_lna) {
@@ -416,21 +461,51 @@ __global__ __launch_bounds__(256) void gla_chunk_scan_kernel(GlaParams P, const 
                                                              const float* __restrict__ lna, int ld_lna,
                                                              const float* __restrict__ U, float* __restrict__ Sin,
                                                              long long u_stride) {
+  constexpr int TB = 128;               // chunk table entries staged at a time
+  __shared__ int last_row[TB], flags[TB];
   const int c0 = blockIdx.x;
-  if (!(chunks[4 * c0 + 3] & 1)) return;  // not the first chunk of its sequence's rows
+  if (!(chunks[4 * c0 + 3] & 1)) return;  // not the first chunk of its sequence's rows (uniform per block)
   const long long per = (long long)P.H * P.D * P.Dv;
   const long long e = (long long)blockIdx.y * 256 + threadIdx.x;
-  if (e >= per) return;
-  const int hd = (int)(e / P.Dv);  // head * D + key channel
+  const bool on = e < per;
+  const int hd = on ? (int)(e / P.Dv) : 0;  // head * D + key channel
   float* st0 = P.state + (long long)chunks[4 * c0 + 2] * P.state_stride;
-  float S = st0[e];
-  for (int c = c0; c < nchunks; ++c) {
-    Sin[(long long)c * u_stride + e] = S;
-    const int r0 = chunks[4 * c], n = chunks[4 * c + 1];
-    S = expf(lna[(long long)(r0 + n - 1) * ld_lna + hd]) * S + U[(long long)c * u_stride + e];
-    if (chunks[4 * c + 3] & 2) break;
+  float S = on ? st0[e] : 0.f;
+  bool done = false;
+  for (int cb = c0; cb < nchunks && !done; cb += TB) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < TB && cb + i < nchunks; i += 256) {
+      last_row[i] = chunks[4 * (cb + i)] + chunks[4 * (cb + i) + 1] - 1;
+      flags[i] = chunks[4 * (cb + i) + 3];
+    }
+    __syncthreads();
+    int cnt = 0;  // chunks of this sequence in the staged part
+    while (cnt < TB && cb + cnt < nchunks) {
+      ++cnt;
+      if (flags[cnt - 1] & 2) {
+        done = true;
+        break;
+      }
+    }
+    if (!on) continue;
+    for (int i0 = 0; i0 < cnt; i0 += 4) {  // the loads do not depend on the state: four chunks' worth in flight
+      float dec[4], u[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int i = min(i0 + k, cnt - 1);
+        dec[k] = lna[(long long)last_row[i] * ld_lna + hd];
+        u[k] = U[(long long)(cb + i) * u_stride + e];
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (i0 + k < cnt) {
+          Sin[(long long)(cb + i0 + k) * u_stride + e] = S;
+          S = expf(dec[k]) * S + u[k];
+        }
+      }
+    }
   }
-  st0[e] = S;
+  if (on) st0[e] = S;
 }
 // outputs of one chunk and head: A is built in LDS first (the exponentials are per pair and channel)
 template <typename T>
@@ -476,12 +551,19 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
 #pragma unroll
   for (int k = 0; k < GC; ++k) acc[k] = 0.f;
   if (g < NG) {
-    for (int i = 0; i < D; ++i) {
-      const float sv = S[(long long)i * Dv + j];
+    for (int i0 = 0; i0 < D; i0 += 8) {  // eight loads of the state's column in flight at a time
+      float sv[8];
 #pragma unroll
-      for (int k = 0; k < GC; ++k) {
-        const int t = g + k * NG;
-        if (t < n) acc[k] += sv * qd[t * D1 + i];
+      for (int u = 0; u < 8; ++u) sv[u] = i0 + u < D ? S[(long long)(i0 + u) * Dv + j] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (i0 + u < D) {
+#pragma unroll
+          for (int k = 0; k < GC; ++k) {
+            const int t = g + k * NG;
+            if (t < n) acc[k] += sv[u] * qd[t * D1 + i0 + u];
+          }
+        }
       }
     }
     for (int sidx = 0; sidx < n; ++sidx) {
@@ -523,9 +605,9 @@ void gla_chunked(const GlaParams& P, const StepRows& R, const GlaChunkWs& W, hip
   const long long per = (long long)HD * P.Dv;
   const dim3 cg(W.nchunks, P.H);
   if (P.f32)
-    hipLaunchKernelGGL(gla_lna_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R.B, W.lna, W.ld_lna);
+    hipLaunchKernelGGL(gla_lna_kernel<float>, dim3(R.B), dim3(256), 0, s, P, R.B, W.lna, W.ld_lna, gla_vec(P));
   else
-    hipLaunchKernelGGL(gla_lna_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R.B, W.lna, W.ld_lna);
+    hipLaunchKernelGGL(gla_lna_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R.B, W.lna, W.ld_lna, gla_vec(P));
   hipLaunchKernelGGL(gla_cum_kernel, dim3(W.nchunks), dim3(256), 0, s, W.chunks, HD, W.lna, W.ld_lna);
   hipLaunchKernelGGL(gla_u_kernel, cg, dim3(256), 0, s, P, W.chunks, W.lna, W.ld_lna, W.U, W.u_stride);
   hipLaunchKernelGGL(gla_chunk_scan_kernel, dim3(W.nchunks, (unsigned)((per + 255) / 256)), dim3(256), 0, s, P, W.chunks,
@@ -632,6 +714,42 @@ void sandwich_add(float* x, const float* y, const float* bias, float sa, const f
     hipLaunchKernelGGL(sandwich_add_kernel<bf16>, dim3(rows), dim3(256), 0, s, x, y, bias, sa, y2, sb, E, g, ls, eps, g_next,
                        (bf16*)hout);
   launched("sandwich_add");
+}
+
+// ------------------------------------------------------------------------------------------------ two output projections
+// C[m][n] = sa * (A1[m] . W1[n] + bias[n]) + sb * (A2[m] . W2[n]) for a few rows (decode steps): one wave per output,
+// both weight rows streamed once per activation row.
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_pair_kernel(const T* __restrict__ A1, int lda1, const T* __restrict__ W1, int K1,
+                                                        const float* __restrict__ bias, float sa, const T* __restrict__ A2,
+                                                        int lda2, const T* __restrict__ W2, int K2, float sb, int M, int N,
+                                                        float* __restrict__ C, int ldc, int v1, int v2) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const float b = bias ? bias[n] : 0.f;
+  for (int m = 0; m < M; ++m) {
+    const float d1 = wave_dot<T>(W1 + (long long)n * K1, A1 + (long long)m * lda1, K1, lane, v1);
+    const float d2 = wave_dot<T>(W2 + (long long)n * K2, A2 + (long long)m * lda2, K2, lane, v2);
+    if (lane == 0) C[(long long)m * ldc + n] = sa * (d1 + b) + sb * d2;
+  }
+}
+void gemv_pair(const void* A1, int lda1, const void* W1, int K1, const float* bias, float sa, const void* A2, int lda2,
+               const void* W2, int K2, float sb, int M, int N, float* C, int ldc, int f32, hipStream_t s) {
+  check(M > 0 && M <= 8 && N > 0 && K1 > 0 && K2 > 0 && A1 && W1 && A2 && W2 && C && lda1 >= K1 && lda2 >= K2 && ldc >= N,
+        "gemv_pair: bad operands (at most 8 rows)");
+  const dim3 grid((N + 3) / 4);
+  if (f32)
+    hipLaunchKernelGGL(gemv_pair_kernel<float>, grid, dim3(256), 0, s, (const float*)A1, lda1, (const float*)W1, K1, bias, sa,
+                       (const float*)A2, lda2, (const float*)W2, K2, sb, M, N, C, ldc,
+                       (int)(vec_ok<float>(A1, lda1, K1) && vec_ok<float>(W1, K1, K1)),
+                       (int)(vec_ok<float>(A2, lda2, K2) && vec_ok<float>(W2, K2, K2)));
+  else
+    hipLaunchKernelGGL(gemv_pair_kernel<bf16>, grid, dim3(256), 0, s, (const bf16*)A1, lda1, (const bf16*)W1, K1, bias, sa,
+                       (const bf16*)A2, lda2, (const bf16*)W2, K2, sb, M, N, C, ldc,
+                       (int)(vec_ok<bf16>(A1, lda1, K1) && vec_ok<bf16>(W1, K1, K1)),
+                       (int)(vec_ok<bf16>(A2, lda2, K2) && vec_ok<bf16>(W2, K2, K2)));
+  launched("gemv_pair");
 }
 
 // ------------------------------------------------------------------------------------------------ gated activation
