@@ -382,7 +382,8 @@ static void launch_gla(const GlaParams& P, const StepRows& R, hipStream_t s) {
     hipLaunchKernelGGL((gla_kernel<T, 64>), grid, dim3(256), 0, s, P, R, gla_vec(P));
 }
 static void check_gla(const GlaParams& P, const StepRows& R) {
-  check(R.B > 0 && P.proj && P.state && P.out && P.a2 && P.a2_b && P.norm_w && P.H > 0 && P.rank > 0 && P.rank <= GLA_MAX_RANK && P.tau > 0.f &&
+  check(R.B > 0 && P.proj && P.state && P.out && P.a2 && P.a2_b && P.norm_w && P.H > 0 && P.rank > 0 && P.rank <= GLA_MAX_RANK &&
+            P.tau > 0.f &&
             gla_supported(P.D, P.Dv),
         "gated linear attention: operands or head sizes (key and value size <= 256, state within the registers)");
 }
@@ -445,7 +446,8 @@ __global__ __launch_bounds__(256) void gla_u_kernel(GlaParams P, const int* __re
     const float Lend = lna[(long long)(r0 + n - 1) * ld_lna + h * D + d], Lt = lna[(long long)(r0 + t) * ld_lna + h * D + d];
     kd[t][d] = P.proj[(long long)(r0 + t) * P.ld + P.off_k + h * D + d] * expf(Lend - Lt);
   }
-  for (int i = tid; i < n * Dv; i += 256) vs[i / Dv][i % Dv] = P.proj[(long long)(r0 + i / Dv) * P.ld + P.off_v + h * Dv + i % Dv];
+  for (int i = tid; i < n * Dv; i += 256)
+    vs[i / Dv][i % Dv] = P.proj[(long long)(r0 + i / Dv) * P.ld + P.off_v + h * Dv + i % Dv];
   __syncthreads();
   const int g = tid / Dv, j = tid % Dv;
   if (g >= NG) return;
@@ -456,59 +458,27 @@ __global__ __launch_bounds__(256) void gla_u_kernel(GlaParams P, const int* __re
     out[(long long)i * Dv + j] = acc;
   }
 }
-// Sin[c] = the state a chunk starts from; the sequence's state after its last chunk goes back to the slot
+// Sin[c] = the state a chunk starts from; the sequence's state after its last chunk goes back to the slot. One thread
+// per state element walks every chunk of the step (a sequence's chunks are consecutive in the table)
 __global__ __launch_bounds__(256) void gla_chunk_scan_kernel(GlaParams P, const int* __restrict__ chunks, int nchunks,
                                                              const float* __restrict__ lna, int ld_lna,
                                                              const float* __restrict__ U, float* __restrict__ Sin,
                                                              long long u_stride) {
-  constexpr int TB = 128;               // chunk table entries staged at a time
-  __shared__ int last_row[TB], flags[TB];
-  const int c0 = blockIdx.x;
-  if (!(chunks[4 * c0 + 3] & 1)) return;  // not the first chunk of its sequence's rows (uniform per block)
-  const long long per = (long long)P.H * P.D * P.Dv;
-  const long long e = (long long)blockIdx.y * 256 + threadIdx.x;
-  const bool on = e < per;
-  const int hd = on ? (int)(e / P.Dv) : 0;  // head * D + key channel
-  float* st0 = P.state + (long long)chunks[4 * c0 + 2] * P.state_stride;
-  float S = on ? st0[e] : 0.f;
-  bool done = false;
-  for (int cb = c0; cb < nchunks && !done; cb += TB) {
-    __syncthreads();
-    for (int i = threadIdx.x; i < TB && cb + i < nchunks; i += 256) {
-      last_row[i] = chunks[4 * (cb + i)] + chunks[4 * (cb + i) + 1] - 1;
-      flags[i] = chunks[4 * (cb + i) + 3];
-    }
-    __syncthreads();
-    int cnt = 0;  // chunks of this sequence in the staged part
-    while (cnt < TB && cb + cnt < nchunks) {
-      ++cnt;
-      if (flags[cnt - 1] & 2) {
-        done = true;
-        break;
-      }
-    }
-    if (!on) continue;
-    for (int i0 = 0; i0 < cnt; i0 += 4) {  // the loads do not depend on the state: four chunks' worth in flight
-      float dec[4], u[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int i = min(i0 + k, cnt - 1);
-        dec[k] = lna[(long long)last_row[i] * ld_lna + hd];
-        u[k] = U[(long long)(cb + i) * u_stride + e];
-      }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        if (i0 + k < cnt) {
-          Sin[(long long)(cb + i0 + k) * u_stride + e] = S;
-          S = expf(dec[k]) * S + u[k];
-        }
-      }
-    }
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long long)P.H * P.D * P.Dv) return;
+  const int hd = (int)(e / P.Dv);  // head * D + key channel
+  float S = 0.f;
+  for (int c = 0; c < nchunks; ++c) {  // the table's entries are the same for every thread: scalar loads
+    const int last = chunks[4 * c] + chunks[4 * c + 1] - 1, slot = chunks[4 * c + 2], flags = chunks[4 * c + 3];
+    float* st_e = P.state + (long long)slot * P.state_stride + e;
+    if (flags & 1) S = *st_e;
+    Sin[c * u_stride + e] = S;
+    S = expf(lna[(long long)last * ld_lna + hd]) * S + U[c * u_stride + e];
+    if (flags & 2) *st_e = S;
   }
-  if (on) st0[e] = S;
 }
 // outputs of one chunk and head: A is built in LDS first (the exponentials are per pair and channel)
-template <typename T>
+template <typename T, int RT>  // RT >= ceil(GC / NG): rows of a column that one thread sums
 __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __restrict__ chunks, const float* __restrict__ lna,
                                                       int ld_lna, const float* __restrict__ Sin, long long u_stride) {
   extern __shared__ float lds[];
@@ -530,11 +500,12 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
   }
   for (int i = tid; i < n * Dv; i += 256) vs[i] = P.proj[(long long)(r0 + i / Dv) * P.ld + P.off_v + h * Dv + i % Dv];
   __syncthreads();
-  for (int p = tid; p < n * n; p += 256) {  // A[t][s], s <= t
-    const int t = p / n, sidx = p % n;
+  for (int p = tid; p < GC * GC; p += 256) {  // A[t][s], s <= t < n; zero elsewhere
+    const int t = p / GC, sidx = p % GC;
     float acc = 0.f;
-    if (sidx <= t)
-      for (int d = 0; d < D; ++d) acc += qd[t * D1 + d] * kk[sidx * D1 + d] * expf(Lc[t * D1 + d] - Lc[sidx * D1 + d]);
+    if (sidx <= t && t < n)
+      for (int d = 0; d < D; ++d)  // exponents <= 0; exp2 on the transcendental unit (1 ulp)
+        acc += qd[t * D1 + d] * kk[sidx * D1 + d] * __builtin_amdgcn_exp2f((Lc[t * D1 + d] - Lc[sidx * D1 + d]) * 1.44269504088896341f);
     A[t * (GC + 1) + sidx] = acc;
   }
   __syncthreads();
@@ -547,9 +518,9 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
   // them whole, the state's column read once per key channel; the rows then meet in LDS for their norms
   const int g = tid / Dv, j = tid % Dv;
   const float* S = Sin + (long long)c * u_stride + (long long)h * D * Dv;
-  float acc[GC];
+  float acc[RT];
 #pragma unroll
-  for (int k = 0; k < GC; ++k) acc[k] = 0.f;
+  for (int k = 0; k < RT; ++k) acc[k] = 0.f;
   if (g < NG) {
     for (int i0 = 0; i0 < D; i0 += 8) {  // eight loads of the state's column in flight at a time
       float sv[8];
@@ -559,9 +530,9 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
       for (int u = 0; u < 8; ++u) {
         if (i0 + u < D) {
 #pragma unroll
-          for (int k = 0; k < GC; ++k) {
-            const int t = g + k * NG;
-            if (t < n) acc[k] += sv[u] * qd[t * D1 + i0 + u];
+          for (int k = 0; k < RT; ++k) {
+            const int t = min(g + k * NG, GC - 1);  // rows past the chunk's end: computed, never stored
+            acc[k] += sv[u] * qd[t * D1 + i0 + u];
           }
         }
       }
@@ -569,9 +540,9 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
     for (int sidx = 0; sidx < n; ++sidx) {
       const float vv = vs[sidx * Dv + j];
 #pragma unroll
-      for (int k = 0; k < GC; ++k) {
-        const int t = g + k * NG;
-        if (t < n && sidx <= t) acc[k] += A[t * (GC + 1) + sidx] * vv;
+      for (int k = 0; k < RT; ++k) {
+        const int t = min(g + k * NG, GC - 1);
+        acc[k] += A[t * (GC + 1) + sidx] * vv;  // A is zero above the diagonal and in rows past the chunk's end
       }
     }
   }
@@ -579,7 +550,7 @@ __global__ __launch_bounds__(256) void gla_out_kernel(GlaParams P, const int* __
   float* ob = vs;   // [GC][Dv]
   if (g < NG) {
 #pragma unroll
-    for (int k = 0; k < GC; ++k) {
+    for (int k = 0; k < RT; ++k) {
       const int t = g + k * NG;
       if (t < n) ob[t * Dv + j] = acc[k];
     }
@@ -610,13 +581,17 @@ void gla_chunked(const GlaParams& P, const StepRows& R, const GlaChunkWs& W, hip
     hipLaunchKernelGGL(gla_lna_kernel<bf16>, dim3(R.B), dim3(256), 0, s, P, R.B, W.lna, W.ld_lna, gla_vec(P));
   hipLaunchKernelGGL(gla_cum_kernel, dim3(W.nchunks), dim3(256), 0, s, W.chunks, HD, W.lna, W.ld_lna);
   hipLaunchKernelGGL(gla_u_kernel, cg, dim3(256), 0, s, P, W.chunks, W.lna, W.ld_lna, W.U, W.u_stride);
-  hipLaunchKernelGGL(gla_chunk_scan_kernel, dim3(W.nchunks, (unsigned)((per + 255) / 256)), dim3(256), 0, s, P, W.chunks,
+  hipLaunchKernelGGL(gla_chunk_scan_kernel, dim3((unsigned)((per + 255) / 256)), dim3(256), 0, s, P, W.chunks,
                      W.nchunks, W.lna, W.ld_lna, W.U, W.Sin, W.u_stride);
   const size_t lds = (size_t)gla_out_lds(P.D, P.Dv) * sizeof(float);
-  if (P.f32)
-    hipLaunchKernelGGL(gla_out_kernel<float>, cg, dim3(256), lds, s, P, W.chunks, W.lna, W.ld_lna, W.Sin, W.u_stride);
-  else
-    hipLaunchKernelGGL(gla_out_kernel<bf16>, cg, dim3(256), lds, s, P, W.chunks, W.lna, W.ld_lna, W.Sin, W.u_stride);
+  const int ng = 256 / P.Dv, rt = (GC + ng - 1) / ng;
+#define GLA_OUT(TT, RT) hipLaunchKernelGGL((gla_out_kernel<TT, RT>), cg, dim3(256), lds, s, P, W.chunks, W.lna, W.ld_lna, W.Sin, W.u_stride)
+  if (P.f32) {
+    if (rt <= 8) GLA_OUT(float, 8); else if (rt <= 16) GLA_OUT(float, 16); else GLA_OUT(float, 32);
+  } else {
+    if (rt <= 8) GLA_OUT(bf16, 8); else if (rt <= 16) GLA_OUT(bf16, 16); else GLA_OUT(bf16, 32);
+  }
+#undef GLA_OUT
   launched("gla_chunked");
 }
 

@@ -49,8 +49,8 @@ def standard():
     key size."""
     return config([(parallel(), glu()),
                    (talking(), None),
-                   (parallel(heads=2, kv_heads=2, dim=8, vdim=20, rot_dims=4, scaling=(), right=gla(heads=3, dim=4, vdim=8, tau=1.0, rank=3)),
-                    glu(24)),
+                   (parallel(heads=2, kv_heads=2, dim=8, vdim=20, rot_dims=4, scaling=(),
+                             right=gla(heads=3, dim=4, vdim=8, tau=1.0, rank=3)), glu(24)),
                    (talking(heads=3, kv_heads=1, dim=12, rot_dims=6, scaling=()), glu(56)),
                    (parallel(heads=3, kv_heads=1, dim=8, vdim=24, rot_dims=8, scaling=("linear", 3.0),
                              right=gla(heads=1, dim=16, vdim=16, tau=16.0, rank=8)), glu(32))])
@@ -85,8 +85,8 @@ def random_config(rng):
         G = rng.choice([1, 2, 4])
         D = rng.choice([32, 48, 64, 96])
         rd, base, sc = rot(D)
-        return parallel(heads=G * rng.choice([1, 2, 4]), kv_heads=G, dim=D, vdim=rng.choice([32, 64, 96]), scale=rng.choice([0.05, 0.1, 0.2]),
-                        rot_dims=rd, base=base, scaling=sc,
+        return parallel(heads=G * rng.choice([1, 2, 4]), kv_heads=G, dim=D, vdim=rng.choice([32, 64, 96]),
+                        scale=rng.choice([0.05, 0.1, 0.2]), rot_dims=rd, base=base, scaling=sc,
                         right=gla(heads=rng.choice([1, 2, 4]), dim=rng.choice([16, 32, 48, 64]), vdim=rng.choice([32, 64, 128]),
                                   tau=rng.choice([1.0, 4.0, 16.0]), rank=rng.choice([4, 16, 32])),
                         left_scale=rng.choice([0.5, 1.0]), right_scale=rng.choice([0.8, 1.5]))

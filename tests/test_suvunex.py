@@ -84,7 +84,8 @@ def test_frequency_scaling_by_hand():
 MECHANISMS = {
     "pair": ([(sc.parallel(), None)], {}),
     "pair_no_rotation_one_kv_head": ([(sc.parallel(heads=3, kv_heads=1, dim=12, vdim=7, rot_dims=0), None)], {}),
-    "pair_all_rotated_linear_scaling": ([(sc.parallel(heads=2, kv_heads=2, dim=8, vdim=8, rot_dims=8, scaling=("linear", 5.0)), None)], {}),
+    "pair_all_rotated_linear_scaling": ([(sc.parallel(heads=2, kv_heads=2, dim=8, vdim=8, rot_dims=8, scaling=("linear", 5.0)),
+                                          None)], {}),
     "pair_one_head_each_wide_values": ([(sc.parallel(heads=1, kv_heads=1, dim=10, vdim=30, rot_dims=4, scaling=(),
                                                       right=sc.gla(heads=1, dim=6, vdim=40, tau=1.0, rank=2)), None)], {}),
     "pair_fast_decay_many_heads": ([(sc.parallel(right=sc.gla(heads=5, dim=4, vdim=4, tau=0.5, rank=7)), None)], {}),
@@ -346,11 +347,11 @@ def test_decays_from_gone_in_a_token_to_kept_for_thousands(tmp_path, device):
 def test_other_sizes(tmp_path, device, dtype):
     """A width, head sizes and a hidden size that are not multiples of 8 (no vector loads), a vocabulary wider than
     a tile, four taps, eps, embedding and logit scales of their own, more key/value heads than one."""
-    layers = [(sc.parallel(heads=6, kv_heads=3, dim=12, vdim=10, scale=0.4, rot_dims=6, right=sc.gla(heads=3, dim=10, vdim=6, tau=2.0, rank=3)),
-               sc.glu(36)),
+    layers = [(sc.parallel(heads=6, kv_heads=3, dim=12, vdim=10, scale=0.4, rot_dims=6,
+                           right=sc.gla(heads=3, dim=10, vdim=6, tau=2.0, rank=3)), sc.glu(36)),
               (sc.talking(heads=6, kv_heads=3, dim=20, scale=0.2, rot_dims=10, scaling=sc.BANDS), sc.glu(20)),
-              (sc.parallel(heads=2, kv_heads=2, dim=64, vdim=64, scale=0.1, rot_dims=32, right=sc.gla(heads=2, dim=32, vdim=64, tau=8.0, rank=16)),
-               None),
+              (sc.parallel(heads=2, kv_heads=2, dim=64, vdim=64, scale=0.1, rot_dims=32,
+                           right=sc.gla(heads=2, dim=32, vdim=64, tau=8.0, rank=16)), None),
               (sc.talking(heads=5, kv_heads=5, dim=6, scale=0.5, rot_dims=2, scaling=()), sc.glu(12))]
     m = sc.Model(tmp_path, sc.config(layers, width=52, vocab=300, eps=1e-3, embed_scale=0.7, taps=4, logit_scale=1.7), seed=17)
     toks = sc.tokens(90, 300, seed=18)
@@ -363,11 +364,11 @@ def test_other_sizes(tmp_path, device, dtype):
 def test_matrix_core_sizes(tmp_path, device):
     """Sizes the matrix-core products and vector loads take (head sizes 64 / 96 / 128), in both dtypes; a prompt portion
     over several tiles and chunks, then single tokens."""
-    layers = [(sc.parallel(heads=6, kv_heads=2, dim=96, vdim=96, scale=0.1, rot_dims=32, base=1e4, right=sc.gla(heads=3, dim=32, vdim=64, tau=8.0, rank=8)),
-               sc.glu(256)),
+    layers = [(sc.parallel(heads=6, kv_heads=2, dim=96, vdim=96, scale=0.1, rot_dims=32, base=1e4,
+                           right=sc.gla(heads=3, dim=32, vdim=64, tau=8.0, rank=8)), sc.glu(256)),
               (sc.talking(heads=6, kv_heads=3, dim=64, scale=0.11, rot_dims=48, base=1e5, scaling=("linear", 2.0)), sc.glu(128)),
-              (sc.parallel(heads=2, kv_heads=2, dim=128, vdim=128, scale=0.09, rot_dims=64, right=sc.gla(heads=2, dim=64, vdim=128, tau=4.0, rank=8)),
-               None)]
+              (sc.parallel(heads=2, kv_heads=2, dim=128, vdim=128, scale=0.09, rot_dims=64,
+                           right=sc.gla(heads=2, dim=64, vdim=128, tau=4.0, rank=8)), None)]
     m = sc.Model(tmp_path, sc.config(layers, width=128, vocab=256), seed=19)
     toks = sc.tokens(200, 256, seed=20)
     want, _ = m.oracle(toks)
