@@ -58,7 +58,7 @@ static void validate_sandwich(const StackExecutor& e, const RunDesc& r, const La
   int n_out = L.heads * L.vdim;
   if (L.r_heads) {
     need(L.a2 && L.a2_b && L.gnorm && L.w_o2 && L.r_rank > 0 && L.r_tau > 0.f && r.state, "gated linear attention operands");
-    need(gla_supported(L.r_dim, L.r_vdim), "gated linear attention head sizes (<= 256, state within the registers)");
+    need(gla_general_supported(L.r_dim, L.r_vdim), "gated linear attention head sizes (<= 256)");
     need_state += (long long)L.r_heads * L.r_dim * L.r_vdim;
     n_out += L.r_heads * L.r_vdim;
   }

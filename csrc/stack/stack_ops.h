@@ -346,7 +346,8 @@ struct GlaParams {
   int f32;
 };
 void gla(const GlaParams& P, const StepRows& R, hipStream_t s);
-bool gla_supported(int D, int Dv);
+bool gla_supported(int D, int Dv);          // the state-in-registers kernel covers these head sizes
+bool gla_general_supported(int D, int Dv);  // the state-in-memory kernel covers the rest, up to 256
 // the same in chunks (prompt portions) over the host-built chunk table of the chunked retention; lna [B][H * D] and
 // U / Sin (one state per chunk) are scratch, raw [B][ld_raw] receives o before its norm
 struct GlaChunkWs {

@@ -381,14 +381,62 @@ static void launch_gla(const GlaParams& P, const StepRows& R, hipStream_t s) {
   else
     hipLaunchKernelGGL((gla_kernel<T, 64>), grid, dim3(256), 0, s, P, R, gla_vec(P));
 }
+// Heads whose state the registers do not hold: the same walk with the state in memory. Thread j owns column j of the
+// state (Dv <= 256 columns), reads and writes it row by row (coalesced over j) and sums its output on the way.
+template <typename T>
+__global__ __launch_bounds__(256) void gla_general_kernel(GlaParams P, StepRows R, int vec) {
+  __shared__ float qs[256], ks[256], as[256], red[4];
+  __shared__ float a1s[GLA_MAX_RANK];
+  const int r0 = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int seq = R.q_seq[r0];
+  if (r0 > 0 && R.q_seq[r0 - 1] == seq) return;  // not the first row of its segment (uniform per block)
+  const int D = P.D, Dv = P.Dv;
+  float* S0 = P.state + (long long)seq * P.state_stride + (long long)h * D * Dv;
+  const float qscale = 1.f / sqrtf((float)D);
+  for (int r = r0; r < R.B && R.q_seq[r] == seq; ++r) {
+    const float* row = P.proj + (long long)r * P.ld;
+    __syncthreads();
+    if (tid < P.rank) a1s[tid] = row[P.off_a1 + tid];
+    if (tid < D) {
+      qs[tid] = row[P.off_q + h * D + tid] * qscale;
+      ks[tid] = row[P.off_k + h * D + tid];
+    }
+    __syncthreads();
+    if (tid < D) as[tid] = expf(gla_ln_alpha<T>(P, a1s, h * D + tid, vec));
+    __syncthreads();
+    float o = 0.f;
+    if (tid < Dv) {
+      const float vj = row[P.off_v + h * Dv + tid];
+      for (int i = 0; i < D; ++i) {
+        const float sv = as[i] * S0[(long long)i * Dv + tid] + ks[i] * vj;
+        S0[(long long)i * Dv + tid] = sv;
+        o += sv * qs[i];
+      }
+    }
+    const float ms = block_sum256(o * o, red) / (float)Dv;
+    if (tid < Dv) {
+      const float y = o / sqrtf(ms + P.eps) * P.norm_w[tid] * silu(row[P.off_g + h * Dv + tid]);
+      st((T*)P.out + (long long)r * P.ld_out + h * Dv + tid, y);
+    }
+  }
+}
+bool gla_general_supported(int D, int Dv) { return D > 0 && Dv > 0 && D <= 256 && Dv <= 256; }
 static void check_gla(const GlaParams& P, const StepRows& R) {
   check(R.B > 0 && P.proj && P.state && P.out && P.a2 && P.a2_b && P.norm_w && P.H > 0 && P.rank > 0 && P.rank <= GLA_MAX_RANK &&
             P.tau > 0.f &&
-            gla_supported(P.D, P.Dv),
-        "gated linear attention: operands or head sizes (key and value size <= 256, state within the registers)");
+            gla_general_supported(P.D, P.Dv),
+        "gated linear attention: operands or head sizes (key and value size <= 256)");
 }
 void gla(const GlaParams& P, const StepRows& R, hipStream_t s) {
   check_gla(P, R);
+  if (!gla_supported(P.D, P.Dv)) {
+    if (P.f32)
+      hipLaunchKernelGGL(gla_general_kernel<float>, dim3(R.B, P.H), dim3(256), 0, s, P, R, gla_vec(P));
+    else
+      hipLaunchKernelGGL(gla_general_kernel<bf16>, dim3(R.B, P.H), dim3(256), 0, s, P, R, gla_vec(P));
+    launched("gla_general");
+    return;
+  }
   if (P.f32)
     launch_gla<float>(P, R, s);
   else

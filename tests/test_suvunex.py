@@ -89,6 +89,7 @@ MECHANISMS = {
     "pair_one_head_each_wide_values": ([(sc.parallel(heads=1, kv_heads=1, dim=10, vdim=30, rot_dims=4, scaling=(),
                                                       right=sc.gla(heads=1, dim=6, vdim=40, tau=1.0, rank=2)), None)], {}),
     "pair_fast_decay_many_heads": ([(sc.parallel(right=sc.gla(heads=5, dim=4, vdim=4, tau=0.5, rank=7)), None)], {}),
+    "pair_state_wider_than_the_registers": ([(sc.parallel(right=sc.gla(heads=1, dim=160, vdim=200, tau=8.0, rank=8)), None)], {}),
     "pair_scales_zero_left": ([(sc.parallel(left_scale=0.0, right_scale=2.0), None)], {}),
     "pair_scales_zero_right": ([(sc.parallel(left_scale=1.5, right_scale=0.0), None)], {}),
     "mixed_heads": ([(sc.talking(), None)], {}),
