@@ -50,6 +50,16 @@ def test_config_roundtrip(std):
     assert std.runner("cpu").w.cfg.layers[0].mixer.right.decay_rank == 5
 
 
+def test_bench_configurations_are_readable():
+    """The sizes `bench.py --stack ... --suvunex` measures are valid configurations of the design."""
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    for z in bench.SUVUNEX_SIZES.values():
+        cfg = bench.suvunex_config(z)
+        assert no_rank(StackConfig.from_suvunex(cfg.to_suvunex())) == no_rank(cfg)
+        assert len(cfg.layers) == 8 and cfg.has_state and sum(s.mixer.talk for s in cfg.layers) == 2
+
+
 def test_unknown_parts_are_refused():
     c = sc.standard().to_suvunex()
     for path, val in ((("layers", 0, "type"), "conv_mixer"), (("layers", 0, "mlp", "kind"), "moe"),
