@@ -315,11 +315,13 @@ void StackExecutor::layer_run_sandwich(int ri, int B, hipStream_t s) {
                  L.ls1, cfg.eps, g_next, h_next, f32, s);
   }
   if (!has_ff) return;
-  {
+  if (B <= 8) {  // decode steps: gate / up projection and activation in one launch
+    gemv_glu(ws.h, E, L.w_ff, E, L.ff, B, ws.hmid, ws.ld_hmid, f32, s);
+  } else {
     GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(g, s);
+    geglu_tanh_cast(ws.proj, ws.ld_proj, B, L.ff, ws.hmid, ws.ld_hmid, f32, s);
   }
-  geglu_tanh_cast(ws.proj, ws.ld_proj, B, L.ff, ws.hmid, ws.ld_hmid, f32, s);
   {
     GemmParams d{ws.hmid, ws.ld_hmid, L.w_dense_down, B, E, L.ff, ws.y, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(d, s);

@@ -371,6 +371,9 @@ void sandwich_add(float* x, const float* y, const float* bias, float sa, const f
 // C[m][n] = sa * (A1[m] . W1[n] + bias[n]) + sb * (A2[m] . W2[n]): two output projections of a few rows (M <= 8) in one launch
 void gemv_pair(const void* A1, int lda1, const void* W1, int K1, const float* bias, float sa, const void* A2, int lda2,
                const void* W2, int K2, float sb, int M, int N, float* C, int ldc, int f32, hipStream_t s);
+// out[m][k] = gelu_tanh(A[m] . W[k]) * (A[m] . W[F + k]), matrix dtype: the gate / up projection of a few rows (M <= 8) with
+// its activation in one launch (W [2F][K]: gate rows, then up rows)
+void gemv_glu(const void* A, int lda, const void* W, int K, int F, int M, void* out, int ld_out, int f32, hipStream_t s);
 // out = gelu_tanh(z[:, :F]) * z[:, F:2F], matrix dtype
 void geglu_tanh_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
 

@@ -775,6 +775,37 @@ void gemv_pair(const void* A1, int lda1, const void* W1, int K1, const float* bi
   launched("gemv_pair");
 }
 
+// ------------------------------------------------------------------------------------------------ gate / up projection + activation
+// out[m][k] = gelu_tanh(A[m] . W[k]) * (A[m] . W[F + k]) for a few rows (decode steps): one wave per hidden unit takes
+// its gate row and its up row, so the activation leaves with the product and needs no launch of its own.
+__device__ __forceinline__ float geglu_tanh(float a, float u) {
+  const float t = tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a));
+  return 0.5f * a * (1.f + t) * u;
+}
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_glu_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W, int K, int F,
+                                                       int M, T* __restrict__ out, int ld_out, int vec) {
+  const int lane = threadIdx.x & 63;
+  const int k = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (k >= F) return;
+  for (int m = 0; m < M; ++m) {
+    const float g = wave_dot<T>(W + (long long)k * K, A + (long long)m * lda, K, lane, vec);
+    const float u = wave_dot<T>(W + (long long)(F + k) * K, A + (long long)m * lda, K, lane, vec);
+    if (lane == 0) st(out + (long long)m * ld_out + k, geglu_tanh(g, u));
+  }
+}
+void gemv_glu(const void* A, int lda, const void* W, int K, int F, int M, void* out, int ld_out, int f32, hipStream_t s) {
+  check(M > 0 && M <= 8 && K > 0 && F > 0 && A && W && out && lda >= K && ld_out >= F, "gemv_glu: bad operands (at most 8 rows)");
+  const dim3 grid((F + 3) / 4);
+  if (f32)
+    hipLaunchKernelGGL(gemv_glu_kernel<float>, grid, dim3(256), 0, s, (const float*)A, lda, (const float*)W, K, F, M, (float*)out,
+                       ld_out, (int)(vec_ok<float>(A, lda, K) && vec_ok<float>(W, K, K)));
+  else
+    hipLaunchKernelGGL(gemv_glu_kernel<bf16>, grid, dim3(256), 0, s, (const bf16*)A, lda, (const bf16*)W, K, F, M, (bf16*)out,
+                       ld_out, (int)(vec_ok<bf16>(A, lda, K) && vec_ok<bf16>(W, K, K)));
+  launched("gemv_glu");
+}
+
 // ------------------------------------------------------------------------------------------------ gated activation
 template <typename T>
 __global__ __launch_bounds__(256) void geglu_tanh_kernel(const float* __restrict__ z, int ld, int rows, int F,
@@ -783,9 +814,7 @@ __global__ __launch_bounds__(256) void geglu_tanh_kernel(const float* __restrict
   if (i >= (long long)rows * F) return;
   const long long r = i / F;
   const int c = (int)(i % F);
-  const float a = z[r * ld + c], u = z[r * ld + F + c];
-  const float t = tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a));
-  st(out + r * ld_out + c, 0.5f * a * (1.f + t) * u);
+  st(out + r * ld_out + c, geglu_tanh(z[r * ld + c], z[r * ld + F + c]));
 }
 void geglu_tanh_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s) {
   check(rows > 0 && F > 0 && z && out && ld >= 2 * F && ld_out >= F, "geglu_tanh_cast: bad operands");
