@@ -24,8 +24,8 @@ import time
 
 import torch
 
-from ..models.config import (BLOCK_POSTNORM, BLOCK_SANDWICH, FF_DENSE, FF_GLU, MIX_ATTENTION, MIX_LATENT, MIX_MAMBA2,
-                             MIX_MLSTM, MIX_RETENTION)
+from ..models.config import (BLOCK_POSTNORM, BLOCK_PRENORM, BLOCK_SANDWICH, FF_DENSE, FF_GLU, MIX_ATTENTION, MIX_LATENT,
+                             MIX_MAMBA2, MIX_MLSTM, MIX_RETENTION)
 from .runner import Runner
 from .weights import StackWeights
 
@@ -53,6 +53,9 @@ class StackExec:
             m, f = spec.mixer, spec.mlp
             if cfg.block == BLOCK_SANDWICH:
                 e.set_layer(i, self._sandwich_layer(L, spec, p))
+                continue
+            if cfg.block == BLOCK_PRENORM:
+                e.set_layer(i, self._prenorm_layer(L, spec, p))
                 continue
             d = dict(kind=m.kind, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale,
                      softcap=m.softcap, qtemp_coef=m.qtemp_coef, qtemp_every=m.qtemp_every, rot_dims=m.rot_dims,
@@ -120,6 +123,25 @@ class StackExec:
                 raise ValueError("a sandwich layer's feed-forward is the gated dense one")
             d.update(ff=f.ff, ff_dense=2, w_ff=p(L["w_ff"]), n_ff=L["n_ff"], w_dense_down=p(L["w_dense_down"]),
                      norm2_w=p(L["norm2"]), norm2_b=p(L["norm2b"]), ls2=p(L["ls2"]))
+        return d
+
+    @staticmethod
+    def _prenorm_layer(L: dict, spec, p) -> dict:
+        """Descriptor of a layer with RMS norms on the inputs of both sublayers (csrc/stack LayerDesc)."""
+        m, f = spec.mixer, spec.mlp
+        d = dict(kind=m.kind, heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim, scale=m.scale, rot_dims=m.rot_dims,
+                 n_in=L["n_in"], w_in=p(L["w_in"]), w_o=p(L["w_o"]), norm_w=p(L["norm_w"]), inv_freq64=p(L["inv_freq64"]),
+                 window=m.window, maps=m.maps, diff=m.diff, lam=L.get("lam", 0.0), gate=int(m.gate), talk=p(L.get("talk")),
+                 score_talk=int(m.score_talk), rot_dim=m.rot_dim, kv_rank=m.kv_rank, dkv_norm=p(L.get("dkv_norm")),
+                 w_uk=p(L.get("w_uk")), w_uvT=p(L.get("w_uvT")), w_ukT=p(L.get("w_ukT")), w_uv=p(L.get("w_uv")),
+                 **{"off_" + k: v for k, v in L["off"].items() if k in ("q", "k", "v", "g", "router")})
+        if f is not None:
+            d.update(norm2_w=p(L["norm2_w"]), w_ff=p(L["w_ff"]), n_ff=L["n_ff"], ff=f.ff)
+            if f.kind == FF_GLU:
+                d.update(ff_dense=3, w_dense_down=p(L["w_dense_down"]))
+            else:
+                d.update(experts=f.experts, top=f.top, w_gu=p(L["w_gu"]), w_down=p(L["w_down"]), group_count=f.group_count,
+                         group_keep=f.group_keep, route_scale=f.route_scale)
         return d
 
     def bind_chunks(self, rows) -> None:
@@ -197,8 +219,12 @@ class StackRunner(Runner):
                 self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
                 ns = cfg.run_state_floats(li)
                 self.states.append(torch.zeros(max_seqs, ns, **f32) if ns else None)
-            elif m.kind == MIX_ATTENTION:
-                self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim, **tt))
+            elif m.kind == MIX_ATTENTION and m.score_talk:  # one K row per token: every key/value head's key side by side
+                self.kc.append(torch.zeros(n_blocks, 1, block_size, m.kv_heads * m.dim, **tt))
+                self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
+                self.states.append(None)
+            elif m.kind == MIX_ATTENTION:                   # (with two maps per head a K row holds [map 1 | map 2])
+                self.kc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.dim * m.maps, **tt))
                 self.vc.append(torch.zeros(n_blocks, m.kv_heads, block_size, m.vdim, **tt))
                 self.states.append(None)
             elif m.kind == MIX_LATENT:  # one row per token: latent | shared rotated key part (the latent is the value too)
@@ -230,7 +256,9 @@ class StackRunner(Runner):
         mam = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_MAMBA2]
         talk = [s.mixer for s in cfg.layers if s.mixer.talk]  # every query head against every key/value head's values
         self.cbuf = torch.zeros(max_batch, (max([m.heads * m.cache_dim for m in lat] + [m.conv_channels for m in mam] +
-                                                [m.heads * m.kv_heads * m.vdim for m in talk], default=1) + 3) // 4 * 4, **f32)
+                                                [m.heads * m.kv_heads * m.vdim for m in talk] +
+                                                [max(m.heads * m.kv_heads * m.dim * m.score_talk, m.heads * m.vdim * m.maps * (m.maps > 1))
+                                                 for m in (s.mixer for s in cfg.layers)], default=1) + 3) // 4 * 4, **f32)
         sandwich = cfg.block == BLOCK_SANDWICH
         self.hn = torch.zeros(max_batch if sandwich else 1, E, **f32)      # normed rows before the input convolution
         self.ybuf2 = torch.zeros(max_batch if sandwich else 1, E, **f32)   # the second mixer's projected output
@@ -261,7 +289,7 @@ class StackRunner(Runner):
         self.scan_ctot = torch.zeros(n_ch, hmax, **f32) if hmax else None
         self.ret_sin = torch.zeros_like(self.ret_u)
         # decode attention over long contexts: partials {maximum, sum, output} of up to 16 splits per (row, head)
-        hv = max([s.mixer.heads * (s.mixer.kv_heads if s.mixer.talk else 1) * (s.mixer.vdim + 2) for s in cfg.layers
+        hv = max([s.mixer.heads * s.mixer.maps * (s.mixer.kv_heads if s.mixer.talk else 1) * (s.mixer.vdim + 2) for s in cfg.layers
                   if s.mixer.kind == MIX_ATTENTION] +
                  [s.mixer.heads * (s.mixer.kv_rank + 2) for s in cfg.layers if s.mixer.kind == MIX_LATENT], default=1)
         self.split_ws = torch.zeros(16 * 16 * hv, **f32)

@@ -414,7 +414,7 @@ class StackWeights:
     def __init__(self, path: str, device: str | torch.device = "cuda", dtype: torch.dtype = torch.bfloat16):
         import os as _os
 
-        from ..models.config import BLOCK_POSTNORM, BLOCK_SANDWICH, MIX_RETENTION, load_stack_config
+        from ..models.config import BLOCK_POSTNORM, BLOCK_PRENORM, BLOCK_SANDWICH, MIX_RETENTION, load_stack_config
         from .safetensors_io import SafetensorsFile
         self.cfg = cfg = self.full_cfg = load_stack_config(path)
         self.device, self.dtype = device, dtype
@@ -440,6 +440,9 @@ class StackWeights:
             p = f"l{i}."
             if cfg.block == BLOCK_SANDWICH:
                 self.layers.append(self._load_sandwich_layer(st, p, spec))
+                continue
+            if cfg.block == BLOCK_PRENORM:
+                self.layers.append(self._load_prenorm_layer(p, spec))
                 continue
             L: dict = dict(norm_w=vec(get(p + "norm1", (E,))), norm_b=vec(get(p + "norm1.b", (E,))))
             if cfg.block == BLOCK_POSTNORM:
@@ -481,6 +484,8 @@ class StackWeights:
             self.layers.append(L)
         if cfg.block == BLOCK_SANDWICH:   # an RMS norm with one number as its weight
             self.final_w, self.final_b = vec(get("final.norm", ())), None
+        elif cfg.block == BLOCK_PRENORM:  # an RMS norm with a weight vector
+            self.final_w, self.final_b = vec(get("final.norm", (E,))), None
         else:
             self.final_w, self.final_b = vec(get("final.norm", (E,))), vec(get("final.norm.b", (E,)))
         self.head = mat(get("head", (V, E)))
@@ -613,6 +618,65 @@ class StackWeights:
             L["ls2"] = vec(get(p + "ls2", (E,)))
             L["w_ff"], L["n_ff"] = mat(get(p + "mlp.gate", (f.ff, E)), get(p + "mlp.up", (f.ff, E))), 2 * f.ff
             L["w_dense_down"] = mat(get(p + "mlp.down", (E, f.ff)))
+        return L
+
+    def _load_prenorm_layer(self, p: str, spec) -> dict:
+        """A layer with RMS norms (weight vectors) on the inputs of both sublayers. The mixer's matrices that read its
+        normed input are one stack `w_in` (attention q | k | v | [gate]; latent attention q | dkv | gate), the
+        feed-forward's are a second stack `w_ff` (gate | up of the dense one, or the router) because it reads the
+        updated stream. Constants that are functions of the weights alone are worked out here in float32: the
+        differential attention's lambda, and the score-mixing matrix with the heads' factors folded in
+        (M[h][g] = talk[h][g] * temp[g]). Rotary frequencies are float64."""
+        from ..models.config import FF_GLU, GATE_ELEMENT, MIX_LATENT, rotary_inv_freq
+        get, mat, vec = self._get, self._mat, self._vec
+        cfg, dev = self.cfg, self.device
+        E, m, f = cfg.n_embd, spec.mixer, spec.mlp
+        H, G, D, Dv = m.heads, m.kv_heads, m.dim, m.vdim
+        L: dict = dict(norm_w=vec(get(p + "norm1", (E,))))
+        if m.kind == MIX_LATENT:
+            C, R = m.kv_rank, m.rot_dim
+            parts = [get(p + "mix.q", (H * (D + R), E)), get(p + "mix.dkv", (C + R, E)), get(p + "mix.g", (H, E))]
+            off = dict(q=0, k=H * (D + R), g=H * (D + R) + C + R)
+            L["dkv_norm"] = vec(get(p + "mix.dkv.norm", (C,)))
+            L["w_uk"] = mat(get(p + "mix.uk", (H * D, C)))
+            L["w_uvT"] = mat(get(p + "mix.uv", (H * Dv, C)).view(H, Dv, C).transpose(1, 2).reshape(H * C, Dv))
+            L["w_ukT"] = mat(get(p + "mix.uk", (H * D, C)).view(H, D, C).transpose(1, 2).reshape(H * C, D))
+            L["w_uv"] = mat(get(p + "mix.uv", (H * Dv, C)))
+        else:
+            parts = [get(p + "mix.q", (m.n_q, E)), get(p + "mix.k", (m.n_k, E)), get(p + "mix.v", (m.n_v, E))]
+            off = dict(q=0, k=m.n_q, v=m.n_q + m.n_k)
+            if m.gate == GATE_ELEMENT:
+                parts.append(get(p + "mix.g", (m.n_out, E)))
+                off["g"] = m.n_q + m.n_k + m.n_v
+            if m.maps == 2:
+                lq1, lk1, lq2, lk2 = (get(p + "mix." + k, (D,)).to(torch.float32) for k in ("lq1", "lk1", "lq2", "lk2"))
+                L["lam"] = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + torch.tensor(m.diff, dtype=torch.float32))
+            if m.score_talk:
+                talk = get(p + "mix.talk", (H, H)).to(torch.float32)
+                temp = get(p + "mix.temp", (H,)).to(torch.float32)
+                L["talk"] = (talk * temp[None, :]).reshape(-1).contiguous().to(dev)
+        L["inv_freq64"] = (torch.tensor(rotary_inv_freq(m.rot_dims, m.rot_base, m.rot_scaling), dtype=torch.float64, device=dev)
+                           if m.rot_dims else None)
+        L["w_in"] = mat(*parts)
+        L["off"], L["n_in"], L["n_ff"] = off, sum(t.shape[0] for t in parts), 0
+        L["w_o"] = mat(get(p + "mix.o", (E, m.n_out)))
+        if f is None:
+            return L
+        L["norm2_w"] = vec(get(p + "norm2", (E,)))
+        if f.kind == FF_GLU:
+            L["w_ff"], L["n_ff"] = mat(get(p + "mlp.gate", (f.ff, E)), get(p + "mlp.up", (f.ff, E))), 2 * f.ff
+            L["w_dense_down"] = mat(get(p + "mlp.down", (E, f.ff)))
+            return L
+        X, F = f.experts, f.ff
+        L["w_ff"], L["n_ff"] = mat(get(p + "mlp.router", (X, E))), X
+        off["router"] = 0
+        gu, dn = [], []
+        for e in range(X):
+            q = f"{p}mlp.e{e}."
+            gu += [get(q + "gate", (F, E)), get(q + "up", (F, E))]
+            dn.append(get(q + "down", (E, F)))
+        L["w_gu"] = mat(*gu).view(X, 2 * F, E)
+        L["w_down"] = mat(*dn).view(X, E, F)
         return L
 
     @property

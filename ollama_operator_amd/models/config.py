@@ -257,13 +257,21 @@ BLOCK_POSTNORM = 1  # x <- x + LN1(mixer(x)), then x <- x + LN2(ff(x)): the norm
 BLOCK_SANDWICH = 2  # x <- x + s1 N1b(mixer(conv_in(N1(x)))), then x <- x + s2 N2b(ff(N2(x))): scalar-weight RMS norms
                     # before and after each sublayer, per-channel scales on the results, a short causal convolution
                     # added to the mixer's input
+BLOCK_PRENORM = 3   # x <- x + mixer(N1(x)), then x <- x + ff(N2(x)): RMS norms with a weight vector on the sublayers' inputs
 
 FF_MOE = 0          # routed experts (+ shared expert)
 FF_DENSE = 1        # W_down act(W_up h), act = relu(z)^2
 FF_GLU = 2          # W_down (act(W_gate h) * (W_up h)), act = the tanh form of gelu
+ACT_GELU_TANH = 0   # activation of a gated dense feed-forward (FF_GLU)
+ACT_RELU = 1
 ROUTE_TOPK_SOFTMAX = 0   # top-k of (logits + bias), softmax over the chosen logits
 ROUTE_SCORE_GROUPS = 1   # softmax over all outputs; choice by score + correction inside the best expert groups;
                          # weights = the chosen scores; trailing outputs may be identity experts
+ROUTE_SIGMOID_GROUPS = 2  # sigmoid scores; a group ranks by the sum of its two largest scores; the chosen scores are
+                          # divided by their sum and multiplied by a constant
+GATE_NONE = 0
+GATE_ELEMENT = 1            # the mixer's output is multiplied element by element with sigmoid(W_g h)
+GATE_HEAD = 2               # one sigmoid gate per head
 
 
 QK_NORM_NONE = 0
@@ -342,14 +350,23 @@ class MixerSpec:
     right: "MixerSpec | None" = None
     left_scale: float = 1.0
     right_scale: float = 1.0
+    # attention options of the pre-norm block's mixers
+    window: int = 0             # > 0: position i sees only j with 0 <= i - j < window
+    maps: int = 1               # 2: differential attention, every head holds two query / key maps [map 1 | map 2] over the
+                                # same values; o = a1 - lambda a2, unit RMS per head, times (1 - diff)
+    diff: float = 0.0           # lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (learned vectors of size dim)
+    gate: int = GATE_NONE       # sigmoid output gate from the mixer's input
+    rot_pairs: bool = False     # the rotation pairs dims (2i, 2i + 1) instead of (i, i + rot_dims / 2)
+    score_talk: bool = False    # the heads' SCORES, each times its own factor, are mixed by a [heads, heads] matrix
+                                # before the softmax
 
     @property
     def n_q(self) -> int:
-        return self.heads * self.dim
+        return self.heads * self.dim * self.maps
 
     @property
     def n_k(self) -> int:
-        return self.kv_heads * self.dim
+        return self.kv_heads * self.dim * self.maps
 
     @property
     def n_v(self) -> int:
@@ -395,6 +412,8 @@ class MoESpec:
     group_count: int = 1        # experts (identity ones included) form this many groups of neighbours
     group_keep: int = 1         # only experts of the best group_keep groups can be chosen
     shared_gate: bool = True    # the shared expert sits behind a scalar sigmoid gate
+    act: int = ACT_GELU_TANH    # FF_GLU: the gate's activation
+    route_scale: float = 1.0    # ROUTE_SIGMOID_GROUPS: factor on the normalised weights
 
     @property
     def n_router(self) -> int:
@@ -721,13 +740,129 @@ class StackConfig:
         return dict(architecture="Suvunex", vocab=self.n_vocab, width=self.n_embd, layers=out, norm=dict(eps=self.norm_eps),
                     embedding=dict(scale=self.embed_scale), canon=dict(taps=self.canon_taps), logit_scale=self.logit_scale)
 
+    # -- config.json of the Dekalorn design
+    @classmethod
+    def from_dekalorn(cls, c: dict) -> "StackConfig":
+        def bad(msg):
+            raise UnsupportedArchitecture("Dekalorn: " + msg)
+
+        def rotary(m: dict, dim: int) -> dict:
+            rot = m.get("rot") or {}
+            sc = rot.get("scaling") or {}
+            scaling = ()
+            if sc:
+                scaling = ("bands", float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
+                if scaling[3] == scaling[2]:
+                    bad("rot.scaling: high and low must differ")
+            dims = int(rot.get("dims", 0))
+            if dims % 2 or dims > dim:
+                bad("rot.dims must be even and at most the rotated size")
+            return dict(rot_dims=dims, rot_base=float(rot.get("base", 10000.0)), rot_scaling=scaling)
+
+        def grouped(m: dict, **kw) -> MixerSpec:
+            mx = MixerSpec(kind=MIX_ATTENTION, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                           dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]),
+                           window=int((m.get("mask") or {}).get("size", 0)), **kw)
+            if min(mx.heads, mx.kv_heads, mx.dim, mx.vdim) <= 0 or mx.heads % mx.kv_heads or mx.window < 0:
+                bad("heads must be a positive multiple of kv_heads")
+            return mx
+
+        layers = []
+        for ent in c["layers"]:
+            m, t = ent["mixer"], ent["type"]
+            if t == "latent_attention":
+                mx = MixerSpec(kind=MIX_LATENT, heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]), vdim=int(m["vdim"]),
+                               scale=float(m["scale"]), rot_dim=int(m["rot_dim"]), kv_rank=int(m["kv_rank"]), gate=GATE_HEAD,
+                               rot_pairs=True, **rotary(m, int(m["rot_dim"])))
+                if min(mx.heads, mx.dim, mx.vdim, mx.kv_rank) <= 0 or mx.rot_dim < 0:
+                    bad("latent attention sizes must be positive")
+            elif t == "attention":
+                mx = grouped(m, maps=2, diff=float(m["diff"]), gate=GATE_ELEMENT)
+            elif t == "attention_2":
+                mx = grouped(m, score_talk=True, rot_pairs=True, **rotary(m, int(m["dim"])))
+            else:
+                raise UnsupportedArchitecture(f"unknown mixer type {t!r}")
+            mlp = None
+            f = ent.get("mlp")
+            if f:
+                kind = f.get("kind")
+                if kind == "dense":
+                    mlp = MoESpec(kind=FF_GLU, ff=int(f["ff"]), act=ACT_RELU)
+                    if mlp.ff <= 0:
+                        bad("mlp.ff must be positive")
+                elif kind == "moe":
+                    r = f["router"]
+                    gr = r.get("groups") or {}
+                    mlp = MoESpec(kind=FF_MOE, route=ROUTE_SIGMOID_GROUPS, experts=int(r["experts"]), top=int(r["top"]),
+                                  ff=int(f["expert"]["ff"]), group_count=int(gr.get("count", 1)),
+                                  group_keep=int(gr.get("keep", gr.get("count", 1))), route_scale=float(r.get("scale", 1.0)),
+                                  shared_gate=False)
+                    if not 0 < mlp.top <= mlp.experts or mlp.ff <= 0:
+                        bad("router: top must be in 1..experts")
+                    if mlp.group_count < 1 or mlp.experts % mlp.group_count or not 0 < mlp.group_keep <= mlp.group_count:
+                        bad("router: groups must divide the experts, keep in 1..count")
+                    if mlp.group_keep * (mlp.experts // mlp.group_count) < mlp.top:
+                        bad("router: the kept groups hold fewer experts than top")
+                else:
+                    raise UnsupportedArchitecture(f"unknown feed-forward kind {kind!r}")
+            layers.append(LayerSpec(mixer=mx, mlp=mlp))
+        loop = c.get("loop") or {}
+        cfg = cls(arch="dekalorn", n_vocab=int(c["vocab"]), n_embd=int(c["width"]), layers=layers,
+                  loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+                  loop_times=int(loop.get("times", 0)) if loop else 0, norm_eps=float(c["norm"]["eps"]), block=BLOCK_PRENORM,
+                  name=str(c.get("name", "")))
+        if cfg.loop_times and not 0 <= cfg.loop_start < cfg.loop_stop <= len(layers):
+            bad("loop: need 0 <= start < stop <= number of layers")
+        return cfg
+
+    def to_dekalorn(self) -> dict:
+        """The config.json this configuration is read from (random-init fixtures, tests)."""
+        def rotary(m: MixerSpec) -> dict:
+            d = dict(base=m.rot_base, dims=m.rot_dims)
+            if m.rot_scaling:
+                _, fa, lo, hi, orig = m.rot_scaling
+                d["scaling"] = dict(factor=fa, low=lo, high=hi, original=orig)
+            return d
+
+        out = []
+        for s in self.layers:
+            m = s.mixer
+            if m.kind == MIX_LATENT:
+                ent = dict(type="latent_attention", mixer=dict(heads=m.heads, dim=m.dim, rot_dim=m.rot_dim, vdim=m.vdim,
+                                                               kv_rank=m.kv_rank, scale=m.scale, rot=rotary(m)))
+            elif m.kind == MIX_ATTENTION and m.maps == 2:
+                ent = dict(type="attention", mixer=dict(heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
+                                                        scale=m.scale, diff=m.diff, mask=dict(size=m.window)))
+            elif m.kind == MIX_ATTENTION and m.score_talk:
+                ent = dict(type="attention_2", mixer=dict(heads=m.heads, kv_heads=m.kv_heads, dim=m.dim, vdim=m.vdim,
+                                                          scale=m.scale, mask=dict(size=m.window), rot=rotary(m)))
+            else:
+                raise UnsupportedArchitecture("Dekalorn has no mixer of this kind")
+            f = s.mlp
+            if f is None:
+                ent["mlp"] = None
+            elif f.kind == FF_GLU:
+                ent["mlp"] = dict(kind="dense", ff=f.ff)
+            else:
+                ent["mlp"] = dict(kind="moe", expert=dict(ff=f.ff),
+                                  router=dict(experts=f.experts, top=f.top, scale=f.route_scale,
+                                              groups=dict(count=f.group_count, keep=f.group_keep)))
+            out.append(ent)
+        c = dict(architecture="Dekalorn", vocab=self.n_vocab, width=self.n_embd, layers=out, norm=dict(eps=self.norm_eps))
+        if self.loop_times:
+            c["loop"] = dict(start=self.loop_start, stop=self.loop_stop, times=self.loop_times)
+        return c
+
     def to_config_json(self) -> dict:
+        if self.arch == "dekalorn":
+            return self.to_dekalorn()
         if self.arch == "suvunex":
             return self.to_suvunex()
         return self.to_norevik() if self.arch == "norevik" else self.to_bizulix()
 
 
-STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix, "Norevik": StackConfig.from_norevik, "Suvunex": StackConfig.from_suvunex}
+STACK_ARCHS = {"Bizulix": StackConfig.from_bizulix, "Norevik": StackConfig.from_norevik, "Suvunex": StackConfig.from_suvunex,
+               "Dekalorn": StackConfig.from_dekalorn}
 
 
 def is_stack_model(path: str) -> bool:

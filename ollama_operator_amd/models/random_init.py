@@ -68,6 +68,8 @@ def write_random_stack(path: str, cfg, seed: int = 0, std: float = 0.05) -> None
         return write_random_norevik(path, cfg, seed=seed)
     if cfg.arch == "suvunex":
         return write_random_suvunex(path, cfg, seed=seed)
+    if cfg.arch == "dekalorn":
+        return write_random_dekalorn(path, cfg, seed=seed)
     g = torch.Generator().manual_seed(seed)
     E, V = cfg.n_embd, cfg.n_vocab
     T: dict = {}
@@ -271,4 +273,73 @@ def write_random_suvunex(path: str, cfg, seed: int = 0) -> None:
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as fh:
         json.dump(cfg.to_suvunex(), fh, indent=1)
+    write_safetensors(os.path.join(path, "model.safetensors"), T)
+
+
+def write_random_dekalorn(path: str, cfg, seed: int = 0) -> None:
+    """Random-init model folder of the Dekalorn design (its tensor names). Projections ~ N(0, 1 / fan-in), queries and
+    keys with a gain so that the softmax is not flat; norm weights near 1; the vectors behind the differential
+    attention's lambda small, so that lambda stays near `diff`; per-head score factors near 1 and a score-mixing matrix
+    near the identity; router matrices wide enough that the chosen experts are not a close call."""
+    import json
+    import os
+
+    import torch
+
+    from ..engine.safetensors_io import write_safetensors
+    from .config import FF_GLU, MIX_LATENT
+    g = torch.Generator().manual_seed(seed)
+    E, V = cfg.n_embd, cfg.n_vocab
+    T: dict = {}
+
+    def rnd(name, shape, s, mean=0.0):
+        T[name] = (mean + s * torch.randn(*shape, generator=g)).to(torch.bfloat16)
+
+    def lin(name, n_out, n_in, gain=1.0):
+        rnd(name, (n_out, n_in), gain / n_in ** 0.5)
+
+    rnd("embed", (V, E), 1.0)
+    if cfg.loop_times:
+        lin("loop.in", E, 2 * E, 1.4)
+    for i, spec in enumerate(cfg.layers):
+        m, f, p = spec.mixer, spec.mlp, f"l{i}."
+        H, G, D, Dv = m.heads, m.kv_heads, m.dim, m.vdim
+        rnd(p + "norm1", (E,), 0.1, 1.0)
+        if m.kind == MIX_LATENT:
+            lin(p + "mix.q", H * (D + m.rot_dim), E, 2.0)
+            lin(p + "mix.dkv", m.kv_rank + m.rot_dim, E, 2.0)
+            rnd(p + "mix.dkv.norm", (m.kv_rank,), 0.1, 1.0)
+            lin(p + "mix.uk", H * D, m.kv_rank, 1.5)
+            lin(p + "mix.uv", H * Dv, m.kv_rank)
+            lin(p + "mix.g", H, E, 1.5)
+        else:
+            lin(p + "mix.q", m.n_q, E, 2.0)
+            lin(p + "mix.k", m.n_k, E, 2.0)
+            lin(p + "mix.v", m.n_v, E)
+            if m.maps == 2:
+                for k in ("lq1", "lk1", "lq2", "lk2"):
+                    rnd(p + "mix." + k, (D,), 0.1)
+                lin(p + "mix.g", H * Dv, E, 1.5)
+            else:
+                T[p + "mix.talk"] = (torch.eye(H) + 0.25 * torch.randn(H, H, generator=g)).to(torch.bfloat16)
+                rnd(p + "mix.temp", (H,), 0.2, 1.0)
+        lin(p + "mix.o", E, H * Dv)
+        if f is None:
+            continue
+        rnd(p + "norm2", (E,), 0.1, 1.0)
+        if f.kind == FF_GLU:
+            lin(p + "mlp.gate", f.ff, E)
+            lin(p + "mlp.up", f.ff, E)
+            lin(p + "mlp.down", E, f.ff)
+            continue
+        for e in range(f.experts):
+            lin(f"{p}mlp.e{e}.gate", f.ff, E)
+            lin(f"{p}mlp.e{e}.up", f.ff, E)
+            lin(f"{p}mlp.e{e}.down", E, f.ff)
+        lin(p + "mlp.router", f.experts, E, 3.0)
+    rnd("final.norm", (E,), 0.1, 1.0)
+    lin("head", V, E)
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as fh:
+        json.dump(cfg.to_dekalorn(), fh, indent=1)
     write_safetensors(os.path.join(path, "model.safetensors"), T)

@@ -477,6 +477,71 @@ def stack_sandwich_add(x, y, g, ls, eps):
     x += ls * stack_scalar_norm(y, g, eps)
 
 
+
+# ---- layers with RMS norms (weight vectors) on the sublayers' inputs (BLOCK_PRENORM): sliding-window attention with two
+# differential maps per head or with scores mixed across the heads, latent attention with a gate per head, a gated dense
+# feed-forward, a sigmoid router with group ranking. One function per kernel of csrc/stack/stack_prenorm.hip.
+
+def stack_rms_norm(x, w, eps):
+    """x / sqrt(mean(x^2) + eps) * w with a weight per coordinate."""
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+
+
+def stack_attention_window(q, kc, vc, block_table, q_seq, q_len, bs, scale, window, k_off, v_head):
+    """q [B, Hq, D] float32. kc [blocks, Gk, bs, Wk]: query head h reads D elements at k_off[h] of the rows of key
+    head h // (Hq // Gk); vc [blocks, Gv, bs, Dv]: it meets the values of head v_head[h]. Row b sees the keys
+    max(0, q_len[b] - window) .. q_len[b] - 1 of its sequence (window 0: all). Returns float32 [B, Hq, Dv]."""
+    B, Hq, D = q.shape
+    Gk = kc.shape[1]
+    out = torch.empty(B, Hq, vc.shape[-1], dtype=torch.float32, device=q.device)
+    for b in range(B):
+        n = int(q_len[b])
+        t = torch.arange(max(0, n - window) if window else 0, n, device=q.device)
+        bt = block_table[int(q_seq[b])].long()
+        kk, vv = kc[bt[t // bs], :, t % bs].float(), vc[bt[t // bs], :, t % bs].float()   # [n, G, W]
+        for h in range(Hq):
+            s = (kk[:, h // (Hq // Gk), k_off[h]:k_off[h] + D] @ q[b, h]) * scale
+            out[b, h] = torch.softmax(s, 0) @ vv[:, v_head[h]]
+    return out
+
+
+def stack_diff_combine(a, lam, diff, eps, gate):
+    """a [B, H, 2, Dv] (the two maps' outputs): (a1 - lam a2) / rms over Dv * (1 - diff) * sigmoid(gate [B, H * Dv])."""
+    B, H, _, Dv = a.shape
+    o = a[:, :, 0] - lam * a[:, :, 1]
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * (1.0 - diff)
+    return o.reshape(B, H * Dv) * torch.sigmoid(gate)
+
+
+def stack_rotate_fold(q, k, pos, inv_freq, mix, groups):
+    """q [B, H, D], k [B, G, D]: adjacent-pair rotation of both, then the queries are folded through the score-mixing
+    matrix: qf[b, h] = [sum over the heads g of key/value head c of mix[h, g] q[b, g], for every c], so that
+    qf[b, h] . [k_0 | ... | k_(G-1)] is head h's mixed score. Returns (qf [B, H, G * D], rotated k [B, G, D])."""
+    B, H, D = q.shape
+    G = k.shape[1]
+    if inv_freq is not None:
+        q, k = stack_rotate_pairs(q, pos, inv_freq), stack_rotate_pairs(k, pos, inv_freq)
+    qf = torch.einsum("hcj,bcjd->bhcd", mix.view(H, G, groups), q.view(B, G, groups, D))
+    return qf.reshape(B, H, G * D), k
+
+
+def stack_route_sigmoid(z, top, group_count, group_keep, scale):
+    """Router logits [B, X] -> sigmoid scores; a group of neighbours ranks by the sum of its two largest scores and
+    only the best `group_keep` groups stay; the `top` largest scores among them (ties: the lower index), divided by
+    their sum (+ 1e-20), times `scale`. Returns expert ids [B, top] int32 and weights [B, top]."""
+    s = torch.sigmoid(z)
+    choice = s
+    if group_count > 1:
+        per = z.shape[1] // group_count
+        best = torch.topk(s.view(-1, group_count, per), min(2, per), dim=-1).values.sum(-1)
+        keep = torch.topk(best, group_keep, dim=-1).indices
+        ok = torch.zeros_like(best, dtype=torch.bool).scatter_(1, keep, True)
+        choice = s.masked_fill(~ok.repeat_interleave(per, dim=1), -1.0)
+    ids = torch.topk(choice, top, dim=-1).indices
+    wt = torch.gather(s, 1, ids)
+    return ids.to(torch.int32), wt / (wt.sum(-1, keepdim=True) + 1e-20) * scale
+
+
 class TorchStackExecutor:
     def __init__(self, runner):
         self.r = runner
@@ -488,9 +553,11 @@ class TorchStackExecutor:
         r.x0[:B] = x
 
     def layer_run(self, ri: int, B: int):
-        from ..models.config import BLOCK_POSTNORM, BLOCK_SANDWICH, MIX_ATTENTION
+        from ..models.config import BLOCK_POSTNORM, BLOCK_PRENORM, BLOCK_SANDWICH, MIX_ATTENTION
         r = self.r
         w, cfg, T = r.w, r.cfg, r.w.dtype
+        if cfg.block == BLOCK_PRENORM:
+            return self.layer_run_prenorm(ri, B)
         if cfg.block == BLOCK_POSTNORM:
             return self.layer_run_postnorm(ri, B)
         if cfg.block == BLOCK_SANDWICH:
@@ -631,6 +698,72 @@ class TorchStackExecutor:
         r.ybuf[:B] = y
         stack_post_norm_add(x, r.ybuf[:B], L["norm2_w"], L["norm2_b"], cfg.norm_eps, idw)
 
+    def layer_run_prenorm(self, ri: int, B: int):
+        """x <- x + mixer(N1(x)), then x <- x + ff(N2(x)), N an RMS norm with a weight vector; a pass of a repeated span
+        opens with x <- W_in [x; x0]."""
+        from ..models.config import FF_GLU, MIX_LATENT
+        r = self.r
+        w, cfg, T = r.w, r.cfg, r.w.dtype
+        li, _ps, opens = r.runs[ri]
+        L, spec = w.layers[li], cfg.layers[li]
+        m, f, off, eps = spec.mixer, spec.mlp, L["off"], cfg.norm_eps
+        H, G, D, Dv, n_out = m.heads, m.kv_heads, m.dim, m.vdim, m.n_out
+        if opens:
+            r.catbuf[:B] = torch.cat([r.resid[:B], r.x0[:B]], 1).to(T)
+            r.resid[:B] = stack_matmul(r.catbuf[:B], w.loop_in)
+        x = r.resid[:B]
+        pos, qseq, qlen, bs = r.d_pos[:B], r.d_qseq[:B], r.d_qlen[:B], r.block_size
+        slot = r.d_slot[:B].long()
+        blk, o = slot // bs, slot % bs
+        r.hbuf[:B] = stack_rms_norm(x, L["norm_w"], eps).to(T)
+        proj = stack_matmul(r.hbuf[:B], L["w_in"])
+        r.proj[:B, :proj.shape[1]] = proj
+        if m.kind == MIX_LATENT:
+            C = m.kv_rank
+            qa = stack_latent_prepare(proj, off, m, dict(L, inv_freq=L["inv_freq64"]), pos, r.d_slot[:B], r.kc[ri], bs, eps)
+            lat = stack_latent_attention(qa, r.kc[ri], C, r.d_block_table, qseq, qlen, bs, m.scale,
+                                         torch.full((H,), -float("inf"), device=qa.device))
+            r.latbuf[:B, :H * C] = lat.reshape(B, H * C).to(T)
+            ov = torch.einsum("bhc,hcv->bhv", r.latbuf[:B, :H * C].float().view(B, H, C), L["w_uvT"].float().view(H, C, Dv))
+            a = (ov * torch.sigmoid(proj[:, off["g"]:off["g"] + H])[:, :, None]).reshape(B, n_out)
+        else:
+            q = proj[:, off["q"]:off["q"] + m.n_q]
+            k = proj[:, off["k"]:off["k"] + m.n_k]
+            r.vc[ri][blk, :, o] = proj[:, off["v"]:off["v"] + m.n_v].view(B, G, Dv).to(T)
+            if m.maps == 2:  # two maps per head: the K pool's rows hold [map 1 | map 2] of a key/value head
+                r.kc[ri][blk, :, o] = k.view(B, G, 2 * D).to(T)
+                a2 = stack_attention_window(q.view(B, 2 * H, D), r.kc[ri], r.vc[ri], r.d_block_table, qseq, qlen, bs, m.scale,
+                                            m.window, [(h % 2) * D for h in range(2 * H)], [h // 2 // (H // G) for h in range(2 * H)])
+                a = stack_diff_combine(a2.view(B, H, 2, Dv), L["lam"], m.diff, eps, proj[:, off["g"]:off["g"] + n_out])
+            else:            # mixed scores: one K row per token holds every key/value head's key side by side
+                qf, kr = stack_rotate_fold(q.view(B, H, D), k.view(B, G, D), pos, L["inv_freq64"], L["talk"].view(H, H), H // G)
+                r.cbuf[:B, :H * G * D] = qf.reshape(B, H * G * D)
+                r.kc[ri][blk, 0, o] = kr.reshape(B, G * D).to(T)
+                a = stack_attention_window(qf, r.kc[ri], r.vc[ri], r.d_block_table, qseq, qlen, bs, m.scale, m.window,
+                                           [0] * H, [h // (H // G) for h in range(H)]).reshape(B, n_out)
+        r.abuf[:B, :n_out] = a.to(T)
+        x += stack_matmul(r.abuf[:B, :n_out], L["w_o"])
+        if f is None:
+            return
+        r.hbuf[:B] = stack_rms_norm(x, L["norm2_w"], eps).to(T)
+        h = r.hbuf[:B]
+        proj = stack_matmul(h, L["w_ff"])
+        r.proj[:B, :proj.shape[1]] = proj
+        if f.kind == FF_GLU:
+            r.hmid[:B, :f.ff] = (torch.relu(proj[:, :f.ff]) * proj[:, f.ff:2 * f.ff]).to(T)
+            x += stack_matmul(r.hmid[:B, :f.ff], L["w_dense_down"])
+            return
+        ids, wt = stack_route_sigmoid(proj[:, :f.experts], f.top, f.group_count, f.group_keep, f.route_scale)
+        r.eids[:B, :f.top], r.ew[:B, :f.top] = ids, wt
+        y = torch.zeros_like(x)
+        for b in range(B):
+            for j in range(f.top):
+                e = int(ids[b, j])
+                gu = stack_matmul(h[b:b + 1], L["w_gu"][e])[0]
+                mid = (F.silu(gu[:f.ff]) * gu[f.ff:]).to(T)
+                y[b] += wt[b, j] * stack_matmul(mid[None], L["w_down"][e])[0]
+        x += y
+
     def layer_run_sandwich(self, ri: int, B: int):
         """x <- x + s1 N1b(mixer(conv_in(N1(x)))), then x <- x + s2 N2b(ff(N2(x)))."""
         r = self.r
@@ -698,6 +831,11 @@ class TorchStackExecutor:
             return
         w, cfg = r.w, r.cfg
         x = r.resid[r.d_logit_idx[:n_logits].long()] if use_idx else r.resid[:n_logits]
+        if cfg.block == 3:  # BLOCK_PRENORM: an RMS norm with a weight vector
+            r.lbuf[:n_logits] = stack_rms_norm(x, w.final_w, cfg.norm_eps).to(w.dtype)
+            z = stack_matmul(r.lbuf[:n_logits], w.head)
+            r.logits[:n_logits, :z.shape[1]] = z
+            return
         if w.final_b is None:  # an RMS norm with one number as its weight, and a plain factor on the logits
             r.lbuf[:n_logits] = stack_scalar_norm(x, w.final_w, cfg.norm_eps).to(w.dtype)
             z = stack_matmul(r.lbuf[:n_logits], w.head) * float(cfg.logit_scale)
