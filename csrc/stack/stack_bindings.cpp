@@ -177,6 +177,13 @@ PYBIND11_MODULE(_stack, m) {
         L.a2_b = Pp<const float>(ptr(d, "a2_b"));
         L.gnorm = Pp<const float>(ptr(d, "gnorm"));
         L.w_o2 = Pp<const void>(ptr(d, "w_o2"));
+        L.window = geti(d, "window");
+        L.maps = geti(d, "maps", 1);
+        L.diff = getf(d, "diff");
+        L.lam = getf(d, "lam");
+        L.gate = geti(d, "gate");
+        L.score_talk = geti(d, "score_talk");
+        L.route_scale = getf(d, "route_scale", 1.f);
         if (L.qtemp_every <= 0) throw std::runtime_error("q_temp.every must be positive");
       })
       .def("set_runs", [](StackExecutor& e, std::vector<py::dict> runs) {

@@ -70,9 +70,41 @@ static void validate_sandwich(const StackExecutor& e, const RunDesc& r, const La
          "gated feed-forward operands");
 }
 
+static void validate_prenorm(const StackExecutor& e, const RunDesc& r, const LayerDesc& L) {
+  const StackWorkspace& ws = e.ws;
+  need(L.norm_w && L.w_in && L.w_o && L.n_in > 0 && L.n_in <= ws.ld_proj, "layer weights missing");
+  need(L.heads * L.vdim <= ws.ld_a, "mixer output wider than its buffer");
+  if (r.opens_pass) need(e.loop_in && ws.cat, "the pass-opening projection is missing");
+  if (L.kind == 2) {
+    need(r.kc && L.w_uk && L.w_uvT && L.dkv_norm && ws.cbuf && ws.lat && L.gate == 2, "latent attention operands");
+    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank + rot_dim <= 256)");
+    need(L.heads * (L.kv_rank + L.rot_dim) <= ws.ld_cbuf && L.heads * L.kv_rank <= ws.ld_lat, "latent attention buffers");
+    need(L.rot_dims == 0 || L.inv_freq64, "latent attention rotary table missing");
+  } else {
+    need(L.kind == 0 && r.kc && r.vc && L.kv_heads > 0 && L.heads % L.kv_heads == 0 && L.window >= 0, "attention run without a K/V pool");
+    need(L.vdim <= 256, "attention value size (<= 256)");
+    if (L.maps == 2) {
+      need(L.dim <= 256 && ws.cbuf && 2 * L.heads * L.vdim <= ws.ld_cbuf && L.gate == 1, "differential attention sizes or buffers");
+    } else {
+      need(L.maps == 1 && L.score_talk && L.talk && ws.cbuf && (long long)L.heads * L.kv_heads * L.dim <= ws.ld_cbuf,
+           "mixed-score attention operands or buffers");
+      need(rotate_fold_supported(L.heads, L.kv_heads, L.dim), "mixed-score attention sizes (kv_heads * dim <= 1024)");
+      need(L.rot_dims % 2 == 0 && L.rot_dims <= L.dim && (L.rot_dims == 0 || L.inv_freq64), "rotary table missing");
+    }
+  }
+  if (L.ff_dense) {
+    need(L.ff_dense == 3 && L.w_ff && L.w_dense_down && L.norm2_w && L.ff > 0 && L.ff <= ws.ld_hmid && 2 * L.ff <= ws.ld_proj && ws.hmid,
+         "gated feed-forward operands");
+  } else if (L.experts) {
+    need(L.w_ff && L.norm2_w && L.n_ff <= ws.ld_proj && L.top > 0 && L.top <= MOE_MAX_TOP && L.top <= ws.ld_top &&
+             L.top * L.ff <= ws.ld_hmid && ws.hmid && ws.eids && ws.ew && L.w_gu && L.w_down && L.experts <= 256,
+         "routed feed-forward operands (up to 256 experts)");
+  }
+}
+
 void StackExecutor::validate() const {
   need(cfg.E > 0 && cfg.V > 0 && cfg.max_B > 0, "not configured");
-  need(embed_w && final_w && (final_b || cfg.block == 2) && head_w, "global weights missing");
+  need(embed_w && final_w && (final_b || cfg.block >= 2) && head_w, "global weights missing");
   need(ws.resid && ws.x0 && ws.h && ws.proj && ws.a && ws.y && ws.lrows, "workspace missing");
   need(in.tokens && in.pos && in.slot && in.q_len && in.q_seq && in.block_table && in.logits, "step inputs missing");
   need(!runs.empty(), "no layer runs");
@@ -81,6 +113,10 @@ void StackExecutor::validate() const {
     const LayerDesc& L = layers[r.layer];
     if (cfg.block == 2) {
       validate_sandwich(*this, r, L);
+      continue;
+    }
+    if (cfg.block == 3) {
+      validate_prenorm(*this, r, L);
       continue;
     }
     need(L.norm_w && L.norm_b && L.w_in && L.w_o && L.n_in > 0 && L.n_in <= ws.ld_proj, "layer weights missing");
@@ -329,7 +365,111 @@ void StackExecutor::layer_run_sandwich(int ri, int B, hipStream_t s) {
   sandwich_add(ws.resid, ws.y, nullptr, 1.f, nullptr, 0.f, B, E, L.norm2_b, L.ls2, cfg.eps, nullptr, nullptr, f32, s);
 }
 
+// x <- x + mixer(N1(x)), then x <- x + ff(N2(x)); N: RMS norm with a weight vector. A pass of a repeated span opens with
+// x <- W_in [x; x0]. Mixers: attention inside a sliding window with two differential maps per head and an
+// element-wise gate; attention inside a sliding window with adjacent-pair rotation and scores mixed across the heads
+// before the softmax; latent attention with one gate per head.
+void StackExecutor::layer_run_prenorm(int ri, int B, hipStream_t s) {
+  const RunDesc& r = runs.at(ri);
+  const LayerDesc& L = layers[r.layer];
+  const int E = cfg.E, f32 = cfg.f32, n_out = L.heads * L.vdim;
+  if (r.opens_pass) {
+    concat_cast(ws.resid, ws.x0, B, E, ws.cat, f32, s);
+    GemmParams g{ws.cat, 2 * E, loop_in, B, E, 2 * E, ws.resid, E, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
+  rms_norm_cast(ws.resid, nullptr, B, E, L.norm_w, cfg.eps, ws.h, f32, s);
+  {  // every matrix that reads the mixer's input, in one product
+    GemmParams g{ws.h, E, L.w_in, B, L.n_in, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  const bool tiled = B > SMALL_B && n_tiles > 0 && tiles;
+  // a window bounds the keys of a decode step: no need to share them among blocks
+  const int splits = L.window > 0 && L.window <= 1024 ? 1 : n_splits;
+  if (L.kind == 2) {
+    const int C = L.kv_rank, W = C + L.rot_dim;
+    LatentParams P{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_g, L.heads, L.dim, L.rot_dim, C, L.vdim, L.rot_dims,
+                   L.inv_freq64, L.dkv_norm, cfg.eps, L.w_uk, L.w_uvT, L.w_ukT, L.w_uv, r.kc, ws.cbuf, ws.ld_cbuf, ws.lat, ws.ld_lat, ws.a,
+                   ws.ld_a, f32, 1};
+    latent_prepare(P, R, s);
+    AttnParams A{ws.cbuf, ws.ld_cbuf, 0, 0, 0, L.heads, 1, W, C, L.scale, 0.f, 0.f, 1, r.kc, r.kc, ws.lat, ws.ld_lat, f32,
+                 n_splits, ws.split_ws, ws.split_ws_floats, W, W, nullptr};
+    if (tiled && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);
+    else
+      attention(A, R, s);
+    latent_expand(P, B, s);
+  } else if (L.maps == 2) {
+    // a K row of a key/value head holds its two maps side by side; the 2 * heads query maps are heads of their own
+    AttnParams St{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, 2 * L.heads, L.kv_heads, 2 * L.dim, L.vdim, L.scale, 0.f, 0.f, 1,
+                  r.kc, r.vc, ws.a, ws.ld_a, f32};
+    attn_prepare(St, R, s);
+    AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, 2 * L.heads, L.kv_heads, L.dim, L.vdim, L.scale, 0.f, 0.f, 1, r.kc,
+                 r.vc, ws.a, ws.ld_a, f32, splits, ws.split_ws, ws.split_ws_floats, 2 * L.dim, 0, nullptr, 0, ws.cbuf, ws.ld_cbuf,
+                 L.window, 2, 0};
+    if (tiled && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);
+    else
+      attention(A, R, s);
+    diff_combine(ws.cbuf, ws.ld_cbuf, B, L.heads, L.vdim, L.lam, L.diff, cfg.eps, ws.proj + L.off_g, ws.ld_proj, ws.a, ws.ld_a, f32, s);
+  } else {
+    RotFoldParams F{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, L.dim, L.vdim, L.rot_dims, L.inv_freq64,
+                    L.talk, r.kc, r.vc, ws.cbuf, ws.ld_cbuf, f32};
+    rotate_fold(F, R, s);
+    // one key row per token serves every head: its width is all key/value heads' keys, the folded queries match it
+    AttnParams A{ws.cbuf, ws.ld_cbuf, 0, 0, 0, L.heads, L.kv_heads, L.kv_heads * L.dim, L.vdim, L.scale, 0.f, 0.f, 1, r.kc, r.vc, ws.a,
+                 ws.ld_a, f32, splits, ws.split_ws, ws.split_ws_floats, 0, 0, nullptr, 0, nullptr, 0, L.window, 1, 1};
+    if (tiled && flash_prefill_supported(A))
+      flash_prefill(A, R, tiles, n_tiles, s);
+    else
+      attention(A, R, s);
+  }
+  {
+    GemmParams o{ws.a, ws.ld_a, L.w_o, B, E, n_out, ws.resid, E, EPI_RESID, 1.f, nullptr, 0.f, f32};
+    gemm(o, s);
+  }
+  if (!L.ff_dense && !L.experts) return;
+  rms_norm_cast(ws.resid, nullptr, B, E, L.norm2_w, cfg.eps, ws.h, f32, s);
+  if (L.ff_dense) {
+    if (B <= 8) {  // decode steps: gate / up projection and activation in one launch
+      gemv_relu_glu(ws.h, E, L.w_ff, E, L.ff, B, ws.hmid, ws.ld_hmid, f32, s);
+    } else {
+      GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+      gemm(g, s);
+      relu_glu_cast(ws.proj, ws.ld_proj, B, L.ff, ws.hmid, ws.ld_hmid, f32, s);
+    }
+    GemmParams d{ws.hmid, ws.ld_hmid, L.w_dense_down, B, E, L.ff, ws.resid, E, EPI_RESID, 1.f, nullptr, 0.f, f32};
+    gemm(d, s);
+    return;
+  }
+  {
+    GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
+    gemm(g, s);
+  }
+  // the experts' weighted outputs are added straight into the stream (y = the stream, y_add)
+  MoeParams M{ws.proj, ws.ld_proj, L.off_router, 0, 0, 0, B, E, L.experts, L.top, L.ff, 0, nullptr, ws.h, L.w_gu, L.w_down, nullptr,
+              ws.eids, ws.ew, ws.ld_top, ws.sgate, ws.hmid, ws.ld_hmid, ws.resid, f32, 0, L.group_count, L.group_keep, ws.idw, 1,
+              L.route_scale};
+  if (B <= SMALL_B && moe_route_sigmoid_fused_supported(M)) {  // decode steps: routing + activations in one launch
+    moe_route_sigmoid_experts(M, s);
+    moe_down(M, s);
+    return;
+  }
+  moe_route_sigmoid(M, s);
+  if (B > SMALL_B && ws.moe.gu && moe_grouped_supported(M)) {
+    moe_grouped(M, ws.moe, s);  // rows sorted by expert, one matrix-core product per expert tile
+  } else {
+    moe_experts(M, s);
+    moe_down(M, s);
+  }
+}
+
 void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
+  if (cfg.block == 3) {
+    layer_run_prenorm(ri, B, s);
+    return;
+  }
   if (cfg.block == 1) {
     layer_run_postnorm(ri, B, s);
     return;
@@ -402,6 +542,12 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
 
 void StackExecutor::head(int n_logits, bool use_idx, hipStream_t s) {
   if (n_logits <= 0) return;
+  if (cfg.block == 3) {  // an RMS norm with a weight vector; plain logits
+    rms_norm_cast(ws.resid, use_idx ? in.logit_idx : nullptr, n_logits, cfg.E, final_w, cfg.eps, ws.lrows, cfg.f32, s);
+    GemmParams g{ws.lrows, cfg.E, head_w, n_logits, cfg.V, cfg.E, in.logits, in.ld_logits, EPI_STORE, 0.f, nullptr, 0.f, cfg.f32};
+    gemm(g, s);
+    return;
+  }
   if (cfg.block == 2) {  // an RMS norm with one number as its weight, and a plain factor on the logits
     scalar_norm_cast(ws.resid, use_idx ? in.logit_idx : nullptr, n_logits, cfg.E, final_w, cfg.eps, ws.lrows, cfg.f32, s);
     GemmParams g{ws.lrows, cfg.E, head_w, n_logits, cfg.V, cfg.E, in.logits, in.ld_logits, EPI_SCALE, cfg.logit_scale, nullptr,

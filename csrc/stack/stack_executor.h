@@ -18,7 +18,8 @@ struct StackConfig {
   int f32 = 0;
   int max_B = 0, max_seqs = 0;
   int block = 0;            // 0: one norm, mixer and feed-forward in parallel; 1: norms on the sublayers' outputs;
-                            // 2: scalar-weight RMS norms before and after both sublayers
+                            // 2: scalar-weight RMS norms before and after both sublayers; 3: RMS norms (weight vectors) on
+                            // the inputs of both sublayers
   float embed_scale = 1.f;
   float logit_scale = 1.f;  // block 2: logits = head x * logit_scale
   int canon_taps = 1;       // block 2: taps of the convolution added to the mixer's input (1: the current token only)
@@ -88,6 +89,14 @@ struct LayerDesc {
   const float* a2_b = nullptr;
   const float* gnorm = nullptr;
   const void* w_o2 = nullptr;       // [E][r_heads * r_vdim]
+  // layers with RMS norms on the sublayers' inputs: norm_w / norm2_w are the weight vectors; ff_dense == 3 is the gated
+  // dense feed-forward with a relu gate; experts use the sigmoid router
+  int window = 0;                   // sliding window of the attention (0: none)
+  int maps = 1;                     // 2: differential attention (two query / key maps per head)
+  float diff = 0.f, lam = 0.f;      // o = (a1 - lam a2) / rms * (1 - diff)
+  int gate = 0;                     // 1: element-wise sigmoid output gate at off_g, 2: one gate per head
+  int score_talk = 0;               // the heads' scores are mixed by `talk` before the softmax
+  float route_scale = 1.f;
 };
 
 struct RunDesc {   // one execution of a layer: its own cache
@@ -171,6 +180,7 @@ class StackExecutor {
   void layer_run(int ri, int B, hipStream_t s);
   void layer_run_postnorm(int ri, int B, hipStream_t s);
   void layer_run_sandwich(int ri, int B, hipStream_t s);
+  void layer_run_prenorm(int ri, int B, hipStream_t s);
   void head(int n_logits, bool use_idx, hipStream_t s);
   void forward(int B, int n_logits, bool use_idx, hipStream_t s);
 };

@@ -536,6 +536,7 @@ void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s) {
 // batch; each head keeps a running maximum and sum; every lane owns value dims lane, lane + 64, ... of every
 // head's output, and a V row is read once for all of them.
 constexpr int ATT_MAXD = 256;
+constexpr int ATT_MAXD_DECODE = 1024;  // the block-per-(row, head) kernel keeps one query in LDS: wide shared key rows fit
 template <typename T>
 __device__ __forceinline__ void load8(const T* p, float* out);
 template <>
@@ -595,7 +596,8 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
 #pragma unroll
     for (int c = 0; c < DC; ++c) acc[r][c] = 0.f;
   }
-  for (int t0 = SPLIT ? 64 * wv : 0; t0 < n; t0 += SPLIT ? 256 : 64) {
+  const int lo = P.window > 0 ? max(0, n - P.window) : 0;  // sliding window: the keys lo .. n - 1
+  for (int t0 = lo + (SPLIT ? 64 * wv : 0); t0 < n; t0 += SPLIT ? 256 : 64) {
     const int t = t0 + lane;
     const bool valid = t < n;
     int rowidx = 0;
@@ -733,7 +735,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttnParams P, StepRows R
 // quarters meet in two lane exchanges. The serial instruction count per wave is what bounds a decode step.
 template <typename T, int DPL>
 __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, StepRows R, int vec, int vvec, int nsplit) {
-  __shared__ __attribute__((aligned(16))) float qs[ATT_MAXD];
+  __shared__ __attribute__((aligned(16))) float qs[ATT_MAXD_DECODE];
   __shared__ float ps[4][64];
   __shared__ int rs[4][64];
   __shared__ float mg[4][2];
@@ -743,7 +745,9 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
   const int vh = P.vheads > 1 ? P.vheads : 1, NH = P.H * vh;
   const int b = blockIdx.x / NH, oh = blockIdx.x % NH, h = oh / vh;
   const int g = h / (P.H / P.G);
-  const int vrow = vh > 1 ? (oh % vh - g) * R.bs : 0;  // from the key's row to the same token's row of the value head
+  const int gv = vh > 1 ? oh % vh : g;           // the value head this output meets
+  const int KG = P.kshared ? 1 : P.G, kg = P.kshared ? 0 : g;  // a shared key row: the K pool has one head
+  const int koff = P.maps > 1 ? (h % P.maps) * P.D : 0;      // several maps per head sit side by side in a K row
   const int split = blockIdx.y;  // long contexts: blockIdx.y-th of nsplit blocks, 64-key groups dealt round robin
   for (int d = threadIdx.x; d < P.D; d += 256) qs[d] = P.proj[(long long)b * P.ld + P.off_q + h * P.D + d];
   const int n = R.q_len[b];
@@ -756,14 +760,16 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
 #pragma unroll
   for (int c = 0; c < DPL; ++c) acc[c] = 0.f;
   __syncthreads();
-  for (int t0 = 64 * (split * 4 + wv); t0 < n; t0 += 256 * nsplit) {
+  const int lo = P.window > 0 ? max(0, n - P.window) : 0;  // sliding window: the keys lo .. n - 1
+  for (int t0 = lo + 64 * (split * 4 + wv); t0 < n; t0 += 256 * nsplit) {
     const int t = t0 + lane;
     const bool valid = t < n;
     int rowidx = 0;
     float dot = 0.f;
     if (valid) {
-      rowidx = (bt[t / R.bs] * P.G + g) * R.bs + t % R.bs;
-      const T* kr = kc + (long long)rowidx * ldk;
+      const int blk = bt[t / R.bs];
+      rowidx = (blk * P.G + gv) * R.bs + t % R.bs;  // the value's row; the key's may sit in a pool of another shape
+      const T* kr = kc + (long long)((blk * KG + kg) * R.bs + t % R.bs) * ldk + koff;
       if (vec) {
         for (int d0 = 0; d0 < P.D; d0 += 64) {
           float k8[8][8];
@@ -794,7 +800,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(AttnParams P, Ste
     l = l * corr + wave_sum(p);
     m = mn;
     ps[wv][lane] = p;
-    rs[wv][lane] = valid ? rowidx + vrow : 0;  // a key past the end: row 0 with weight 0
+    rs[wv][lane] = valid ? rowidx : 0;  // a key past the end: row 0 with weight 0
 #pragma unroll
     for (int c = 0; c < DPL; ++c) acc[c] *= corr;
     __builtin_amdgcn_wave_barrier();
@@ -919,7 +925,7 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(AttnParams P, int 
 template <typename T>
 static void launch_attention_decode(const AttnParams& P, const StepRows& R, hipStream_t s) {
   const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
-  const int vec = P.D % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;
+  const int vec = P.D % 8 == 0 && ldk % 8 == 0 && ((uintptr_t)P.kc & 15) == 0;  // (a map's offset is a multiple of D)
   const int NH = P.H * (P.vheads > 1 ? P.vheads : 1);
   const int ns = (P.nsplit > 1 && P.split_ws && (long long)R.B * NH * P.nsplit * (P.Dv + 2) <= P.split_ws_floats) ? P.nsplit : 1;
   dim3 grid(R.B * NH, ns);
@@ -1001,10 +1007,14 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   const int row0 = tiles[2 * blockIdx.x], nrows = tiles[2 * blockIdx.x + 1];
   const int vh = P.vheads > 1 ? P.vheads : 1;  // output heads: (query head, value head) pairs with vheads = G
   const int oh = blockIdx.y, h = oh / vh, g = h / (P.H / P.G), gv = vh > 1 ? oh % vh : g;
+  const int KG = P.kshared ? 1 : P.G, kg = P.kshared ? 0 : g;  // a shared key row: the K pool has one head
+  const int koff = P.maps > 1 ? (h % P.maps) * D : 0;        // several maps per head sit side by side in a K row
   const int* bt = R.block_table + (long long)R.q_seq[row0] * R.max_blocks;
   const int qrow = row0 + min(q, nrows - 1);
   const int qlen = q < nrows ? R.q_len[qrow] : 0;
+  const int kfirst = P.window > 0 ? qlen - P.window : 0;     // sliding window: this lane's query sees keys kfirst .. qlen - 1
   const int kmax = R.q_len[row0 + nrows - 1];
+  const int kmin = P.window > 0 ? max(0, R.q_len[row0] - P.window) & ~31 : 0;  // the first key any row of the tile sees
   // queries: B operand, lane (q, hf) holds dims 16 kk + 8 hf + 0..7
   bf16x8 qhi[KD], qlo[KD];
   {
@@ -1043,8 +1053,8 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
   auto fetch = [&](int t0) {
     {
       const int key = min(t0 + kperm, kmax - 1);
-      const long long rowidx = (long long)(bt[key / R.bs] * P.G + g) * R.bs + key % R.bs;
-      const uint16_t* kr = kc + rowidx * ldk + 8 * hf;
+      const long long rowidx = (long long)(bt[key / R.bs] * KG + kg) * R.bs + key % R.bs;
+      const uint16_t* kr = kc + rowidx * ldk + koff + 8 * hf;
 #pragma unroll
       for (int kk = 0; kk < KD; ++kk) kf_n[kk] = *(const u32x4*)(kr + 16 * kk);
     }
@@ -1056,8 +1066,8 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
       vs_n[i] = *(const u32x4*)(vc + rowidx * ldv + 8 * seg);
     }
   };
-  fetch(0);
-  for (int t0 = 0; t0 < kmax; t0 += 32) {
+  fetch(kmin);
+  for (int t0 = kmin; t0 < kmax; t0 += 32) {
     u32x4 kf_c[KD], vs_c[VPL];
 #pragma unroll
     for (int kk = 0; kk < KD; ++kk) kf_c[kk] = kf_n[kk];
@@ -1090,7 +1100,8 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
     for (int r = 0; r < 16; ++r) {
       float sc = sacc[r] * P.scale;
       if (P.softcap != 0.f) sc = P.softcap * fast_tanh(sc * inv_cap);
-      const bool vis = t0 + 16 * (r >> 3) + 8 * hf + (r & 7) < qlen;
+      const int key = t0 + 16 * (r >> 3) + 8 * hf + (r & 7);
+      const bool vis = key < qlen && key >= kfirst;
       pr[r] = vis ? sc : -1e30f;
       mx = fmaxf(mx, pr[r]);
     }
@@ -1158,14 +1169,15 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
 }
 // (key size / 16, value size / 32) the kernel is built for: equal key and value sizes 64 / 96 / 128, and the rows of
 // latent attention (key = latent + shared rotated part, value = the latent)
-#define FLASH_SHAPES(X) X(4, 2) X(6, 3) X(8, 4) X(7, 3) X(8, 3) X(9, 4) X(10, 4) X(12, 5) X(14, 6) X(16, 6) X(16, 7)
+#define FLASH_SHAPES(X) \
+  X(4, 2) X(6, 3) X(8, 4) X(7, 3) X(8, 3) X(9, 4) X(10, 4) X(12, 5) X(14, 6) X(16, 6) X(16, 7) X(2, 2) X(4, 4) X(12, 2) X(16, 2) X(16, 4)
 bool flash_prefill_supported(const AttnParams& P) {
   bool shape = false;
 #define FLASH_HAS(KD, NV) shape |= P.D == 16 * KD && P.Dv == 32 * NV;
   FLASH_SHAPES(FLASH_HAS)
 #undef FLASH_HAS
   const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
-  return !P.f32 && shape && ldk % 8 == 0 && ldv % 8 == 0 && P.ld % 4 == 0 && P.off_q % 4 == 0 && (P.H * P.D) % 4 == 0 &&
+  return !P.f32 && shape && ldk % 8 == 0 && ldv % 8 == 0 && (P.maps <= 1 || P.H % P.maps == 0) && P.ld % 4 == 0 && P.off_q % 4 == 0 && (P.H * P.D) % 4 == 0 &&
          ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
 }
 void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {
@@ -1181,11 +1193,14 @@ void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int
   launched("flash_prefill");
 }
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
-  check(R.B > 0 && P.D > 0 && P.D <= ATT_MAXD && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 && P.H % P.G == 0 && (P.out || P.out32) &&
-            (P.vheads <= 1 || P.vheads == P.G),
-        "attention: head sizes up to 256, heads a multiple of key/value heads");
-  // decode steps (and short portions): a block per (row, head); so are float32 outputs and (query head, value head) pairs
-  if (R.B * P.H <= 1024 || P.out32 || P.vheads > 1) {
+  // a block per (row, head) serves decode steps (and short portions), float32 outputs, (query head, value head) pairs,
+  // several maps per head and a shared key row (whose width may pass 256)
+  const bool per_head = R.B * P.H <= 1024 || P.out32 || P.vheads > 1 || P.maps > 1 || P.kshared;
+  check(R.B > 0 && P.D > 0 && P.D <= (per_head ? ATT_MAXD_DECODE : ATT_MAXD) && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 &&
+            P.H % P.G == 0 && (P.out || P.out32) && (P.vheads <= 1 || P.vheads == P.G) && P.window >= 0 &&
+            (P.maps <= 1 || P.H % (P.G * P.maps) == 0),
+        "attention: head sizes up to 256 (a shared key row up to 1024), heads a multiple of key/value heads");
+  if (per_head) {
     if (P.f32)
       launch_attention_decode<float>(P, R, s);
     else
@@ -1647,7 +1662,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeParams P, int vec, int
   }
   if (P.Fs > 0)
     y += P.sgate[b] * wave_dot<T>((const T*)P.sh_down + (long long)n * P.Fs, hm + P.top * P.F, P.Fs, lane, vec_s != 0);
-  if (lane == 0) P.y[(long long)b * P.E + n] = y;
+  if (lane == 0) P.y[(long long)b * P.E + n] = P.y_add ? P.y[(long long)b * P.E + n] + y : y;
 }
 // ---- prompt portions: pairs (row, routed expert) sorted by expert, one matrix-core product per expert tile
 // One block: counts per expert (LDS atomics hand every pair its rank inside its expert; the order inside an
@@ -1696,11 +1711,11 @@ __global__ __launch_bounds__(256) void moe_act_kernel(const float* __restrict__ 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ ds,
                                                           const int* __restrict__ inv, const float* __restrict__ ew,
                                                           int ld_top, const float* __restrict__ sgate, int B, int E, int top,
-                                                          int shared) {
+                                                          int shared, int y_add) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= (long long)B * E) return;
   const int b = (int)(i / E), n = (int)(i % E);
-  float acc = shared ? sgate[b] * y[i] : 0.f;
+  float acc = shared ? sgate[b] * y[i] : y_add ? y[i] : 0.f;  // (y_add: y is the residual stream, no shared expert)
   float routed = 0.f;
   for (int j = 0; j < top; ++j) routed += ew[(long long)b * ld_top + j] * ds[(long long)inv[b * top + j] * E + n];
   y[i] = routed + acc;
@@ -1710,7 +1725,7 @@ bool moe_grouped_supported(const MoeParams& P) {
          P.ld_hmid % 8 == 0));
 }
 void moe_grouped(const MoeParams& P, const MoeGroupWs& W, hipStream_t s) {
-  check(moe_grouped_supported(P) && W.rank && W.srow && W.inv && W.tiles && W.ntiles && W.gu && W.hs && W.ds,
+  check(moe_grouped_supported(P) && W.rank && W.srow && W.inv && W.tiles && W.ntiles && W.gu && W.hs && W.ds && !(P.y_add && P.Fs > 0),
         "grouped routed feed-forward: workspace or sizes");
   const int pairs = P.B * P.top;
   const int tile_m = pairs / P.X >= 192 ? 128 : 64;
@@ -1761,7 +1776,7 @@ void moe_grouped(const MoeParams& P, const MoeGroupWs& W, hipStream_t s) {
   {
     const long long n = (long long)P.B * P.E;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, P.y, W.ds, W.inv, P.ew, P.ld_top,
-                       P.sgate, P.B, P.E, P.top, (int)(P.Fs > 0));
+                       P.sgate, P.B, P.E, P.top, (int)(P.Fs > 0), P.y_add);
     launched("moe_combine");
   }
 }
@@ -1873,7 +1888,7 @@ __global__ __launch_bounds__(256) void moe_down_out_kernel(MoeParams P, const T*
     if (lane == 0) x[(long long)b * P.E + n] += mult * y;
   }
 }
-static void check_moe(const MoeParams& P);
+static void check_moe(const MoeParams& P, bool bias = true);
 template <typename T>
 static void launch_moe_fused(const MoeParams& P, const void* a, int lda, const void* w_o, int Ko, float* x, float mult,
                              hipStream_t s) {
@@ -1898,9 +1913,9 @@ void moe_fused_small(const MoeParams& P, const void* a, int lda, const void* w_o
   launched("moe_fused_small");
 }
 
-static void check_moe(const MoeParams& P) {
+static void check_moe(const MoeParams& P, bool bias) {  // bias: the caller reads router_b
   check(P.B > 0 && P.X > 0 && P.top > 0 && P.top <= P.X + P.identity && P.top <= MOE_MAX_TOP && P.F > 0 && P.proj && P.h && P.w_gu &&
-            P.w_down && P.eids && P.ew && P.hmid && P.y && P.router_b && P.ld_top >= P.top &&
+            P.w_down && P.eids && P.ew && P.hmid && P.y && (P.router_b || !bias) && P.ld_top >= P.top &&
             P.ld_hmid >= P.top * P.F + P.Fs && (P.Fs == 0 || (P.sh_down && P.sgate)),
         "routed feed-forward: bad operands (top <= 16)");
 }
@@ -1913,7 +1928,7 @@ void moe_route(const MoeParams& P, hipStream_t s) {
   launched("moe_route");
 }
 void moe_experts(const MoeParams& P, hipStream_t s) {
-  check_moe(P);
+  check_moe(P, false);
   dim3 grid((P.F + 3) / 4, P.B * P.top);
   if (P.f32)
     hipLaunchKernelGGL(moe_experts_kernel<float>, grid, dim3(256), 0, s, P,
@@ -1932,7 +1947,7 @@ static void launch_moe_down(const MoeParams& P, hipStream_t s) {
   hipLaunchKernelGGL(moe_down_kernel<T>, grid, dim3(256), 0, s, P, v, vs);
 }
 void moe_down(const MoeParams& P, hipStream_t s) {
-  check_moe(P);
+  check_moe(P, false);
   if (P.f32)
     launch_moe_down<float>(P, s);
   else

@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void latent_expand_kernel(LatentParams P, int 
     const int i = idx >> 6, col = blockIdx.z * 64 + (idx & 63);
     if (col < Dv) {
       const float o = part[0][i][idx & 63] + part[1][i][idx & 63] + part[2][i][idx & 63] + part[3][i][idx & 63];
-      const float g = P.proj[(long long)(r0 + i) * P.ld + P.off_g + h * Dv + col];
+      const float g = P.proj[(long long)(r0 + i) * P.ld + P.off_g + (P.gate_heads ? h : h * Dv + col)];
       st((T*)P.out + (long long)(r0 + i) * P.ld_out + h * Dv + col, o * sigmoidf(g));
     }
   }
@@ -297,7 +297,8 @@ __global__ __launch_bounds__(256) void latent_expand_small_kernel(LatentParams P
   const T* w = (const T*)P.w_uv + (long long)item * P.C;
   for (int b = 0; b < B; ++b) {
     const float v = wave_dot<T>(w, (const T*)P.lat + (long long)b * P.ld_lat + h * P.C, P.C, lane, vec != 0);
-    if (lane == 0) st((T*)P.out + (long long)b * P.ld_out + item, v * sigmoidf(P.proj[(long long)b * P.ld + P.off_g + item]));
+    if (lane == 0)
+      st((T*)P.out + (long long)b * P.ld_out + item, v * sigmoidf(P.proj[(long long)b * P.ld + P.off_g + (P.gate_heads ? h : item)]));
   }
 }
 bool latent_supported(int D, int R, int C, int Dv) {

@@ -79,6 +79,14 @@ struct AttnParams {
   int vheads;
   float* out32;         // non-null: the outputs leave in float32 here (row stride ld_out32) instead of `out`
   int ld_out32;
+  int window;           // > 0: a row sees only its last `window` keys (itself included)
+  // maps = M > 1: H counts M query maps per head, laid out [head][map]; a K row of key/value head g holds the M key maps
+  // side by side (row stride ldk >= M * D) and query map h reads elements (h % M) * D ...; all maps of a head meet the
+  // same values. Output "head" h is query map h.
+  int maps;
+  // kshared: the K pool has ONE head whose row (D wide) serves every query head, while the V pool keeps its G heads
+  // (query head h meets the values of head h / (H / G)): scores that are sums over all key/value heads
+  int kshared;
 };
 // q *= 1 + coef * ln(floor((pos + 1) / every) + 1); k, v of every row stored at its slot
 void attn_prepare(const AttnParams& P, const StepRows& R, hipStream_t s);
@@ -153,6 +161,8 @@ struct MoeParams {
   // router_b is the choice correction; idw [B] receives the summed weight of the chosen identity outputs
   int identity, group_count, group_keep;
   float* idw;
+  int y_add;            // moe_down / moe_grouped: y += the feed-forward's output (y = the residual stream) instead of y =
+  float route_scale;    // sigmoid router (moe_route_sigmoid): factor on the normalised weights
 };
 void moe_route(const MoeParams& P, hipStream_t s);   // top-k ids + softmax weights, shared gate and activation
 // softmax over all router outputs, choice by score + correction inside the best expert groups, weights = the
@@ -213,6 +223,7 @@ struct LatentParams {
   void* out;            // [B][ld_out] matrix dtype: (W_uv_h lat_h) * sigmoid(g), head-major
   int ld_out;
   int f32;
+  int gate_heads;       // 1: the gate is one number per head ([H] at off_g) instead of one per output element
 };
 void latent_prepare(const LatentParams& P, const StepRows& R, hipStream_t s);
 void latent_expand(const LatentParams& P, int B, hipStream_t s);
@@ -376,6 +387,46 @@ void gemv_pair(const void* A1, int lda1, const void* W1, int K1, const float* bi
 void gemv_glu(const void* A, int lda, const void* W, int K, int F, int M, void* out, int ld_out, int f32, hipStream_t s);
 // out = gelu_tanh(z[:, :F]) * z[:, F:2F], matrix dtype
 void geglu_tanh_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
+
+
+// ---- layers with RMS norms (weight vectors) on the inputs of both sublayers (stack_prenorm.hip)
+// out[r] = x[idx ? idx[r] : r] / rms * w, matrix dtype
+void rms_norm_cast(const float* x, const int* idx, int rows, int E, const float* w, float eps, void* out, int f32, hipStream_t s);
+// differential attention: o32 [B][ld_o] holds per head the two maps' outputs side by side ([H][2][Dv], float32);
+// out[b][h] = (a1 - lam a2) / rms over Dv * (1 - diff) * sigmoid(gate[b][h * Dv ...]) (gate null: no gate), matrix dtype
+void diff_combine(const float* o32, int ld_o, int B, int H, int Dv, float lam, float diff, float eps, const float* gate, int ld_gate,
+                  void* out, int ld_out, int f32, hipStream_t s);
+// attention whose scores are mixed across the heads before the softmax, score_h = sum_g mix[h][g] (q_g . k_c(g)):
+// q and k turn in adjacent pairs (2i, 2i + 1), i < rot_dims / 2, by pos * inv_freq[i]; the K pool's row of a token is
+// [k_0 | ... | k_(G-1)] (one head, G * D wide), the V pool is [blocks][G][bs][Dv]; the queries leave folded through the
+// mixing matrix, qf[b][h] = [sum_(g of head c) mix[h][g] q_g, for c < G], so that attention over the shared key row
+// with H query heads of width G * D gives the mixed scores
+struct RotFoldParams {
+  const float* proj;    // [B][ld] float32: q [H][D] at off_q, k [G][D] at off_k, v [G][Dv] at off_v
+  int ld, off_q, off_k, off_v;
+  int H, G, D, Dv;
+  int rot_dims;
+  const double* inv_freq;  // [rot_dims / 2]
+  const float* mix;     // [H][H]
+  void* kc;             // [blocks][1][bs][G * D]
+  void* vc;             // [blocks][G][bs][Dv]
+  float* qf;            // [B][ld_qf]: [H][G * D]
+  int ld_qf;
+  int f32;
+};
+void rotate_fold(const RotFoldParams& P, const StepRows& R, hipStream_t s);
+bool rotate_fold_supported(int H, int G, int D);
+// out = relu(z[:, :F]) * z[:, F:2F], matrix dtype
+void relu_glu_cast(const float* z, int ld, int rows, int F, void* out, int ld_out, int f32, hipStream_t s);
+// out[m][k] = relu(A[m] . W[k]) * (A[m] . W[F + k]), matrix dtype: gate / up projection of a few rows (M <= 16) + activation
+void gemv_relu_glu(const void* A, int lda, const void* W, int K, int F, int M, void* out, int ld_out, int f32, hipStream_t s);
+// sigmoid scores; a group of neighbours ranks by the sum of its two largest scores, only the best group_keep groups
+// stay; the `top` largest scores, divided by their sum, times route_scale -> eids / ew, as moe_route leaves them, so
+// moe_experts, moe_down and moe_grouped follow unchanged (no shared expert, no router bias)
+void moe_route_sigmoid(const MoeParams& P, hipStream_t s);
+// a few rows (decode steps): the same routing and the routed activations (moe_experts' work) in one launch
+void moe_route_sigmoid_experts(const MoeParams& P, hipStream_t s);
+bool moe_route_sigmoid_fused_supported(const MoeParams& P);
 
 }  // namespace stack
 }  // namespace omx
