@@ -377,6 +377,42 @@ SUVUNEX_SIZES = {
 }
 
 
+# the Dekalorn design at the same widths: windowed attention with two differential maps per head, windowed attention
+# with scores mixed across the heads, latent attention, in turn; the first feed-forward is dense, the others route 2 of 8
+# experts (4 groups, the best 2 kept)
+DEKALORN_SIZES = {
+    "s": dict(E=1024, pattern="dtldtldt", diff=(8, 4, 64, 128, 1024), talk=(16, 4, 64, 64, 512), lat=(16, 64, 32, 64, 192),
+              F=512, X=8, top=2, dense=2048),
+    "m": dict(E=2048, pattern="dtldtldt", diff=(16, 4, 128, 128, 1024), talk=(16, 2, 128, 128, 512), lat=(16, 128, 64, 128, 192),
+              F=1024, X=8, top=2, dense=4096),
+}
+
+
+def dekalorn_config(z: dict, vocab: int = 32000):
+    """A Dekalorn model with the sizes of a real model's layers (random weights)."""
+    from ollama_operator_amd.models.config import (ACT_RELU, BLOCK_PRENORM, FF_GLU, FF_MOE, GATE_ELEMENT, GATE_HEAD, MIX_ATTENTION,
+                                                    MIX_LATENT, ROUTE_SIGMOID_GROUPS, LayerSpec, MixerSpec, MoESpec, StackConfig)
+    layers = []
+    for i, c in enumerate(z["pattern"]):
+        if c == "d":
+            h, g, d, dv, w = z["diff"]
+            m = MixerSpec(kind=MIX_ATTENTION, heads=h, kv_heads=g, dim=d, vdim=dv, scale=d ** -0.5, window=w, maps=2, diff=0.5,
+                          gate=GATE_ELEMENT)
+        elif c == "t":
+            h, g, d, dv, w = z["talk"]
+            m = MixerSpec(kind=MIX_ATTENTION, heads=h, kv_heads=g, dim=d, vdim=dv, scale=d ** -0.5, window=w, score_talk=True,
+                          rot_pairs=True, rot_dims=d, rot_base=1e6, rot_scaling=("bands", 8.0, 1.0, 4.0, 8192.0))
+        else:
+            h, d, r, dv, rank = z["lat"]
+            m = MixerSpec(kind=MIX_LATENT, heads=h, kv_heads=1, dim=d, vdim=dv, rot_dim=r, kv_rank=rank, scale=(d + r) ** -0.5,
+                          rot_dims=r, rot_base=1e4, gate=GATE_HEAD, rot_pairs=True)
+        f = (MoESpec(kind=FF_GLU, ff=z["dense"], act=ACT_RELU) if i == 0 else
+             MoESpec(kind=FF_MOE, route=ROUTE_SIGMOID_GROUPS, experts=z["X"], top=z["top"], ff=z["F"], group_count=4, group_keep=2,
+                     route_scale=2.0, shared_gate=False))
+        layers.append(LayerSpec(mixer=m, mlp=f))
+    return StackConfig(arch="dekalorn", n_vocab=vocab, n_embd=z["E"], layers=layers, norm_eps=1e-6, block=BLOCK_PRENORM)
+
+
 def suvunex_config(z: dict, vocab: int = 32000):
     """A Suvunex model with the sizes of a real model's layers (random weights)."""
     from ollama_operator_amd.models.config import (BLOCK_SANDWICH, FF_GLU, MIX_ATTENTION, MIX_GLA, QK_NORM_UNIT_LAST,
@@ -509,6 +545,15 @@ def bench_stack(a) -> None:
             out[name]["suvunex_bf16"] = measure(r)
             out[name]["suvunex_weights_gb"] = round(r.w.nbytes / 1e9, 3)
             r.close()
+        if a.dekalorn:  # the Dekalorn design at the same width and depth, through the same engine and measurement
+            d = os.path.join(a.dir, f"dekalorn-{name}")
+            if not os.path.exists(os.path.join(d, "model.safetensors")):
+                write_random_stack(d, dekalorn_config(DEKALORN_SIZES[name]), seed=0)
+            r = StackRunner(d, device="cuda:0", dtype="bfloat16", max_batch=a.chunk, max_seqs=2, ctx=ctx)
+            r.warmup()
+            out[name]["dekalorn_bf16"] = measure(r)
+            out[name]["dekalorn_weights_gb"] = round(r.w.nbytes / 1e9, 3)
+            r.close()
         if not a.stack_only:
             cfg = ModelConfig(name=f"mixtral-like-{name}", n_vocab=32000, n_embd=z["E"], n_layer=len(z["pattern"]),
                               n_head=z["H"], n_head_kv=z["G"], n_ff=z["F"], n_rot=z["D"], n_embd_head=z["D"],
@@ -536,6 +581,8 @@ def main():
     ap.add_argument("--no-bizulix", action="store_true", help="with --stack: skip the Bizulix model (profiles of one design)")
     ap.add_argument("--suvunex", action="store_true", help="with --stack: also measure the Suvunex design (attention with "
                     "sinks beside gated linear attention, mixed-heads attention, input convolutions) at the same widths")
+    ap.add_argument("--dekalorn", action="store_true", help="with --stack: also measure the Dekalorn design (windowed "
+                    "differential and mixed-score attention, latent attention, sigmoid-routed experts) at the same widths")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--tp", type=int, default=1, help="tensor-parallel degree: one sequence sharded over T GPUs")
     ap.add_argument("--allow-shared", action="store_true",

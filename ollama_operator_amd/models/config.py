@@ -754,7 +754,7 @@ class StackConfig:
                 scaling = ("bands", float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"]))
                 if scaling[3] == scaling[2]:
                     bad("rot.scaling: high and low must differ")
-            dims = int(rot.get("dims", 0))
+            dims = int(rot.get("dims", dim if rot else 0))
             if dims % 2 or dims > dim:
                 bad("rot.dims must be even and at most the rotated size")
             return dict(rot_dims=dims, rot_base=float(rot.get("base", 10000.0)), rot_scaling=scaling)

@@ -31,7 +31,9 @@ def silu(z):
 
 def rotary_frequencies(rot):
     """f_i = base^(-2i / dims); with `scaling`, by wavelength bands: short waves kept, long waves divided by
-    `factor`, a linear blend in between."""
+    `factor`, a linear blend in between. No `rot`, or no dims: nothing turns."""
+    if not rot or not rot.get("dims"):
+        return torch.zeros(0, dtype=F64)
     dims = rot["dims"]
     f = [rot["base"] ** (-2.0 * i / dims) for i in range(dims // 2)]
     sc = rot.get("scaling")
@@ -52,13 +54,13 @@ def rotary_frequencies(rot):
 
 def rotate_pairs(x, pos, freqs):
     """x [n, ..., D]: dims (2i, 2i + 1), i < len(freqs), of the last axis turn by pos * freqs[i]; the rest pass."""
+    n, m = x.shape[0], freqs.numel()
+    ang = pos.to(F64)[:, None] * freqs[None, :]
+    ang = ang.view(n, *([1] * (x.dim() - 2)), m)
+    u, v = x[..., 0:2 * m:2], x[..., 1:2 * m:2]
     out = x.clone()
-    for t in range(x.shape[0]):
-        for i in range(freqs.numel()):
-            a = float(pos[t]) * float(freqs[i])
-            u, v = x[t, ..., 2 * i], x[t, ..., 2 * i + 1]
-            out[t, ..., 2 * i] = u * math.cos(a) - v * math.sin(a)
-            out[t, ..., 2 * i + 1] = v * math.cos(a) + u * math.sin(a)
+    out[..., 0:2 * m:2] = u * torch.cos(ang) - v * torch.sin(ang)
+    out[..., 1:2 * m:2] = v * torch.cos(ang) + u * torch.sin(ang)
     return out
 
 
@@ -85,7 +87,7 @@ def latent_attention(h, W, m, eps):
     q = (h @ W["q"].T).view(n, H, D + R)
     dkv = h @ W["dkv"].T
     c = rms_norm(dkv[:, :C], W["dkv.norm"], eps)
-    fr = rotary_frequencies(m["rot"])
+    fr = rotary_frequencies(m.get("rot"))
     kr = rotate_pairs(dkv[:, C:], pos, fr)                 # [n, R]
     qr = rotate_pairs(q[..., D:], pos, fr)                 # [n, H, R]
     ku = (c @ W["uk"].T).view(n, H, D)
@@ -108,7 +110,7 @@ def differential_attention(h, W, m, eps):
     k = (h @ W["k"].T).view(n, G, 2, D)
     v = (h @ W["v"].T).view(n, G, Dv)
     lam = math.exp(float((W["lq1"] * W["lk1"]).sum())) - math.exp(float((W["lq2"] * W["lk2"]).sum())) + diff
-    ok = visible(n, m["mask"]["size"])
+    ok = visible(n, (m.get("mask") or {}).get("size", 0))
     out = torch.zeros(n, H, Dv, dtype=F64)
     for hd in range(H):
         g = hd // (H // G)
@@ -124,13 +126,13 @@ def mixed_score_attention(h, W, m, eps):
     n = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     pos = torch.arange(n)
-    fr = rotary_frequencies(m["rot"])
+    fr = rotary_frequencies(m.get("rot"))
     q = rotate_pairs((h @ W["q"].T).view(n, H, D), pos, fr)
     k = rotate_pairs((h @ W["k"].T).view(n, G, D), pos, fr)
     v = (h @ W["v"].T).view(n, G, Dv)
     s = torch.stack([(q[:, hd] @ k[:, hd // (H // G)].T) * m["scale"] * W["temp"][hd] for hd in range(H)])   # [H, n, n]
     s = torch.einsum("hg,gij->hij", W["talk"], s)
-    ok = visible(n, m["mask"]["size"])
+    ok = visible(n, (m.get("mask") or {}).get("size", 0))
     out = torch.stack([masked_softmax(s[hd], ok) @ v[:, hd // (H // G)] for hd in range(H)], 1)
     return out.reshape(n, H * Dv) @ W["o"].T
 
