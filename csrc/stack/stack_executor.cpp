@@ -379,8 +379,16 @@ void StackExecutor::layer_run_prenorm(int ri, int B, hipStream_t s) {
     gemm(g, s);
   }
   StepRows R{B, in.pos, in.slot, in.q_len, in.q_seq, in.block_table, in.max_blocks, in.bs};
-  rms_norm_cast(ws.resid, nullptr, B, E, L.norm_w, cfg.eps, ws.h, f32, s);
-  {  // every matrix that reads the mixer's input, in one product
+  const bool fused_in = gemv_ln_supported(B, E, f32);
+  // differential attention: a K row of a key/value head holds its two maps side by side, so the K/V store sees heads
+  // of 2 * dim
+  AttnParams St{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, L.heads, L.kv_heads, 2 * L.dim, L.vdim, L.scale, 0.f, 0.f, 1,
+                r.kc, r.vc, ws.a, ws.ld_a, f32};
+  if (fused_in) {  // decode steps: norm + every matrix that reads the mixer's input (+ that K/V store) in one launch
+    gemv_ln(ws.resid, E, L.norm_w, nullptr, cfg.eps, L.w_in, B, L.n_in, ws.proj, ws.ld_proj, ws.h,
+            L.kind == 0 && L.maps == 2 ? &St : nullptr, &R, f32, s);
+  } else {
+    rms_norm_cast(ws.resid, nullptr, B, E, L.norm_w, cfg.eps, ws.h, f32, s);
     GemmParams g{ws.h, E, L.w_in, B, L.n_in, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(g, s);
   }
@@ -401,10 +409,8 @@ void StackExecutor::layer_run_prenorm(int ri, int B, hipStream_t s) {
       attention(A, R, s);
     latent_expand(P, B, s);
   } else if (L.maps == 2) {
-    // a K row of a key/value head holds its two maps side by side; the 2 * heads query maps are heads of their own
-    AttnParams St{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, 2 * L.heads, L.kv_heads, 2 * L.dim, L.vdim, L.scale, 0.f, 0.f, 1,
-                  r.kc, r.vc, ws.a, ws.ld_a, f32};
-    attn_prepare(St, R, s);
+    // the 2 * heads query maps are heads of their own
+    if (!fused_in) attn_prepare(St, R, s);
     AttnParams A{ws.proj, ws.ld_proj, L.off_q, L.off_k, L.off_v, 2 * L.heads, L.kv_heads, L.dim, L.vdim, L.scale, 0.f, 0.f, 1, r.kc,
                  r.vc, ws.a, ws.ld_a, f32, splits, ws.split_ws, ws.split_ws_floats, 2 * L.dim, 0, nullptr, 0, ws.cbuf, ws.ld_cbuf,
                  L.window, 2, 0};
@@ -430,7 +436,11 @@ void StackExecutor::layer_run_prenorm(int ri, int B, hipStream_t s) {
     gemm(o, s);
   }
   if (!L.ff_dense && !L.experts) return;
-  rms_norm_cast(ws.resid, nullptr, B, E, L.norm2_w, cfg.eps, ws.h, f32, s);
+  if (L.experts && fused_in) {  // decode steps: norm + router in one launch (the normed rows leave for the experts)
+    gemv_ln(ws.resid, E, L.norm2_w, nullptr, cfg.eps, L.w_ff, B, L.n_ff, ws.proj, ws.ld_proj, ws.h, nullptr, nullptr, f32, s);
+  } else {
+    rms_norm_cast(ws.resid, nullptr, B, E, L.norm2_w, cfg.eps, ws.h, f32, s);
+  }
   if (L.ff_dense) {
     if (B <= 8) {  // decode steps: gate / up projection and activation in one launch
       gemv_relu_glu(ws.h, E, L.w_ff, E, L.ff, B, ws.hmid, ws.ld_hmid, f32, s);
@@ -443,7 +453,7 @@ void StackExecutor::layer_run_prenorm(int ri, int B, hipStream_t s) {
     gemm(d, s);
     return;
   }
-  {
+  if (!fused_in) {
     GemmParams g{ws.h, E, L.w_ff, B, L.n_ff, E, ws.proj, ws.ld_proj, EPI_STORE, 0.f, nullptr, 0.f, f32};
     gemm(g, s);
   }

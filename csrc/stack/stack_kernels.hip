@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ A,
   }
 }
 
-// ---- decode steps: layer norm + input projection (+ the attention layer's query temperature and K/V store)
+// ---- decode steps: layer norm (nb null: RMS norm) + input projection (+ the attention layer's query temperature and K/V store)
 // Every block normalises the step's few rows again (they are E floats each) into LDS, rounded to the matrix
 // dtype as the unfused path stores them, then its four waves take one weight row each. Block 0 also writes the
 // normed rows out for the routed experts. QkvEpi: outputs in the q range are multiplied by the row's query
@@ -104,10 +104,10 @@ __global__ __launch_bounds__(256) void gemv_ln_kernel(const float* __restrict__ 
       const int i = tid + 256 * j;
       xr[j] = i < E ? row[i] : 0.f;
       gw[j] = i < E ? nw[i] : 0.f;
-      gb[j] = i < E ? nb[i] : 0.f;
+      gb[j] = (nb && i < E) ? nb[i] : 0.f;
       sum += xr[j];
     }
-    const float mean = block_sum256(sum, red) / (float)E;
+    const float mean = nb ? block_sum256(sum, red) / (float)E : 0.f;  // no bias vector: an RMS norm, nothing is centred
     float sq = 0.f;
 #pragma unroll
     for (int j = 0; j < LN_XR; ++j) {
@@ -211,7 +211,7 @@ bool gemv_ln_supported(int M, int E, int f32) {
 }
 void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps, const void* W, int M, int N, float* C,
              int ldc, void* hout, const AttnParams* A, const StepRows* R, int f32, hipStream_t s) {
-  check(gemv_ln_supported(M, E, f32) && x && nw && nb && W && C && hout && N > 0 && ldc >= N, "gemv_ln: bad operands");
+  check(gemv_ln_supported(M, E, f32) && x && nw && W && C && hout && N > 0 && ldc >= N, "gemv_ln: bad operands");
   QkvEpi q{};
   if (A) {
     check(R && R->pos && R->slot && A->kc && A->vc, "gemv_ln: attention epilogue without rows or pools");

@@ -99,7 +99,8 @@ void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int
 bool flash_prefill_supported(const AttnParams& P);
 constexpr int FLASH_TILE_ROWS = 32;
 
-// decode steps (M <= 8 rows that fit LDS): C = layer_norm(x) . W^T in one launch; the normed rows also go to hout
+// decode steps (M <= 8 rows that fit LDS): C = layer_norm(x) . W^T in one launch (nb null: the norm is an RMS norm with
+// weight nw, x / sqrt(mean(x^2) + eps) * nw); the normed rows also go to hout
 // (matrix dtype). With A (an attention layer): q outputs get the row's query temperature, k and v outputs are
 // also stored at the row's cache slot, so no attn_prepare follows.
 void gemv_ln(const float* x, int E, const float* nw, const float* nb, float eps, const void* W, int M, int N, float* C,
