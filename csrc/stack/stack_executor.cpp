@@ -16,7 +16,7 @@ static void validate_postnorm(const StackExecutor& e, const RunDesc& r, const La
   need(ws.ret.ld_o >= L.heads * L.vdim && ws.ret.obuf, "mixer output wider than its float32 buffer");
   if (L.kind == 2) {
     need(r.kc && L.w_uk && L.w_uvT && L.dkv_norm && L.sink && ws.cbuf && ws.lat, "latent attention operands");
-    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank + rot_dim <= 256)");
+    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank <= 256, kv_rank + rot_dim <= 1024)");
     need(L.heads * (L.kv_rank + L.rot_dim) <= ws.ld_cbuf && L.heads * L.kv_rank <= ws.ld_lat, "latent attention buffers");
     need(L.rot_dims == 0 || L.inv_freq64, "latent attention rotary table missing");
   } else if (L.kind == 3) {
@@ -77,14 +77,15 @@ static void validate_prenorm(const StackExecutor& e, const RunDesc& r, const Lay
   if (r.opens_pass) need(e.loop_in && ws.cat, "the pass-opening projection is missing");
   if (L.kind == 2) {
     need(r.kc && L.w_uk && L.w_uvT && L.dkv_norm && ws.cbuf && ws.lat && L.gate == 2, "latent attention operands");
-    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank + rot_dim <= 256)");
+    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim),
+         "latent attention sizes (dim <= 256, kv_rank <= 256, kv_rank + rot_dim <= 1024)");
     need(L.heads * (L.kv_rank + L.rot_dim) <= ws.ld_cbuf && L.heads * L.kv_rank <= ws.ld_lat, "latent attention buffers");
     need(L.rot_dims == 0 || L.inv_freq64, "latent attention rotary table missing");
   } else {
     need(L.kind == 0 && r.kc && r.vc && L.kv_heads > 0 && L.heads % L.kv_heads == 0 && L.window >= 0, "attention run without a K/V pool");
     need(L.vdim <= 256, "attention value size (<= 256)");
     if (L.maps == 2) {
-      need(L.dim <= 256 && ws.cbuf && 2 * L.heads * L.vdim <= ws.ld_cbuf && L.gate == 1, "differential attention sizes or buffers");
+      need(L.dim <= 1024 && ws.cbuf && 2 * L.heads * L.vdim <= ws.ld_cbuf && L.gate == 1, "differential attention sizes or buffers");
     } else {
       need(L.maps == 1 && L.score_talk && L.talk && ws.cbuf && (long long)L.heads * L.kv_heads * L.dim <= ws.ld_cbuf,
            "mixed-score attention operands or buffers");

@@ -1195,7 +1195,7 @@ void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int
 void attention(const AttnParams& P, const StepRows& R, hipStream_t s) {
   // a block per (row, head) serves decode steps (and short portions), float32 outputs, (query head, value head) pairs,
   // several maps per head and a shared key row (whose width may pass 256)
-  const bool per_head = R.B * P.H <= 1024 || P.out32 || P.vheads > 1 || P.maps > 1 || P.kshared;
+  const bool per_head = R.B * P.H <= 1024 || P.out32 || P.vheads > 1 || P.maps > 1 || P.kshared || P.D > ATT_MAXD;
   check(R.B > 0 && P.D > 0 && P.D <= (per_head ? ATT_MAXD_DECODE : ATT_MAXD) && P.Dv > 0 && P.Dv <= ATT_MAXD && P.G > 0 &&
             P.H % P.G == 0 && (P.out || P.out32) && (P.vheads <= 1 || P.vheads == P.G) && P.window >= 0 &&
             (P.maps <= 1 || P.H % (P.G * P.maps) == 0),

@@ -302,12 +302,14 @@ __global__ __launch_bounds__(256) void latent_expand_small_kernel(LatentParams P
   }
 }
 bool latent_supported(int D, int R, int C, int Dv) {
-  return D > 0 && D <= LAT_MAXD && R >= 0 && C > 0 && C <= LAT_MAXC && Dv > 0 && C + R <= 256;
+  // the latent is the attention's value (up to 256 wide); the cached row [latent | rotated part] is its key: up to 256 on
+  // every attention kernel, up to 1024 on the block-per-(row, head) kernel alone
+  return D > 0 && D <= LAT_MAXD && R >= 0 && C > 0 && C <= 256 && Dv > 0 && C + R <= 1024;
 }
 static void check_latent(const LatentParams& P) {
   check(P.proj && P.cache && P.qa && P.lat && P.out && P.w_uk && P.w_uvT && P.norm_w &&
             latent_supported(P.D, P.R, P.C, P.Dv) && P.rot_dims % 2 == 0 && P.rot_dims <= P.R && (P.rot_dims == 0 || P.inv_freq),
-        "latent attention: operands or sizes (dim <= 256, kv_rank <= 512, kv_rank + rot_dim <= 256)");
+        "latent attention: operands or sizes (dim <= 256, kv_rank <= 256, kv_rank + rot_dim <= 1024)");
 }
 constexpr int LAT_SMALL = 8;  // steps of at most this many rows take the wave-per-output kernels
 void latent_prepare(const LatentParams& P, const StepRows& R, hipStream_t s) {

@@ -418,6 +418,21 @@ def test_other_sizes(tmp_path, device, dtype):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+def test_wide_key_rows(tmp_path, device):
+    """Key rows wider than 256: a latent row of 200 + 120, a shared key row of 4 x 80 and of 8 x 64, maps of 72; only the
+    kernel with one block per (row, head) holds such a query, also for a prompt portion of many rows."""
+    layers = [(dc.latent(heads=2, dim=24, rot_dim=120, vdim=16, kv_rank=200, scale=0.1, base=1e4), None),
+              (dc.talk(heads=4, kv_heads=4, dim=80, vdim=24, scale=0.1, rot_dims=40, base=1e4, window=90), dc.dense()),
+              (dc.talk(heads=8, kv_heads=8, dim=64, vdim=8, scale=0.1, rot_dims=64, base=1e3, scaling=(), window=33), None),
+              (dc.diff(heads=2, kv_heads=1, dim=72, vdim=40, scale=0.1, window=100), None)]
+    m = dc.Model(tmp_path, dc.config(layers, width=64, vocab=80), seed=27)
+    toks = dc.tokens(300, 80, seed=28)
+    want, _ = m.oracle(toks)
+    r = m.runner(device, max_batch=512, kv_tokens=320)
+    dc.check(dc.run_cuts(r, toks, [280] + list(range(281, 301)))[250:], want[250:], "float32", "wide key rows")
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_matrix_core_sizes(tmp_path, device):
     """Sizes the matrix-core products and vector loads take (map sizes 32 and 64, shared key rows of 192 and 256, a
     latent row of 160), in both dtypes; a prompt portion over several tiles and windows, then single tokens."""
