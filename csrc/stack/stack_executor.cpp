@@ -16,7 +16,8 @@ static void validate_postnorm(const StackExecutor& e, const RunDesc& r, const La
   need(ws.ret.ld_o >= L.heads * L.vdim && ws.ret.obuf, "mixer output wider than its float32 buffer");
   if (L.kind == 2) {
     need(r.kc && L.w_uk && L.w_uvT && L.dkv_norm && L.sink && ws.cbuf && ws.lat, "latent attention operands");
-    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim), "latent attention sizes (dim <= 256, kv_rank <= 256, kv_rank + rot_dim <= 1024)");
+    need(latent_supported(L.dim, L.rot_dim, L.kv_rank, L.vdim),
+         "latent attention sizes (dim <= 256, kv_rank <= 256, kv_rank + rot_dim <= 1024)");
     need(L.heads * (L.kv_rank + L.rot_dim) <= ws.ld_cbuf && L.heads * L.kv_rank <= ws.ld_lat, "latent attention buffers");
     need(L.rot_dims == 0 || L.inv_freq64, "latent attention rotary table missing");
   } else if (L.kind == 3) {

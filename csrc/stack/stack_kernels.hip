@@ -1170,14 +1170,16 @@ __global__ __launch_bounds__(64) void flash_prefill_kernel(AttnParams P, StepRow
 // (key size / 16, value size / 32) the kernel is built for: equal key and value sizes 64 / 96 / 128, and the rows of
 // latent attention (key = latent + shared rotated part, value = the latent)
 #define FLASH_SHAPES(X) \
-  X(4, 2) X(6, 3) X(8, 4) X(7, 3) X(8, 3) X(9, 4) X(10, 4) X(12, 5) X(14, 6) X(16, 6) X(16, 7) X(2, 2) X(4, 4) X(12, 2) X(16, 2) X(16, 4)
+  X(4, 2) X(6, 3) X(8, 4) X(7, 3) X(8, 3) X(9, 4) X(10, 4) X(12, 5) X(14, 6) X(16, 6) X(16, 7) \
+  X(2, 2) X(4, 4) X(12, 2) X(16, 2) X(16, 4)
 bool flash_prefill_supported(const AttnParams& P) {
   bool shape = false;
 #define FLASH_HAS(KD, NV) shape |= P.D == 16 * KD && P.Dv == 32 * NV;
   FLASH_SHAPES(FLASH_HAS)
 #undef FLASH_HAS
   const int ldk = P.ldk ? P.ldk : P.D, ldv = P.ldv ? P.ldv : P.Dv;
-  return !P.f32 && shape && ldk % 8 == 0 && ldv % 8 == 0 && (P.maps <= 1 || P.H % P.maps == 0) && P.ld % 4 == 0 && P.off_q % 4 == 0 && (P.H * P.D) % 4 == 0 &&
+  return !P.f32 && shape && ldk % 8 == 0 && ldv % 8 == 0 && (P.maps <= 1 || P.H % P.maps == 0) && P.ld % 4 == 0 &&
+         P.off_q % 4 == 0 && (P.H * P.D) % 4 == 0 &&
          ((uintptr_t)P.proj & 15) == 0 && ((uintptr_t)P.kc & 15) == 0 && ((uintptr_t)P.vc & 15) == 0;
 }
 void flash_prefill(const AttnParams& P, const StepRows& R, const int* tiles, int ntiles, hipStream_t s) {

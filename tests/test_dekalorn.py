@@ -407,8 +407,10 @@ def test_other_sizes(tmp_path, device, dtype):
     """A width, head sizes and hidden sizes that are not multiples of 8 (no vector loads), a vocabulary wider than a
     tile, an eps of its own, three query heads per key/value head, more groups than kept, a span in the middle."""
     layers = [(dc.diff(heads=6, kv_heads=2, dim=12, vdim=10, scale=0.4, lam=0.45, window=29), dc.dense(36)),
-              (dc.talk(heads=6, kv_heads=3, dim=20, vdim=14, scale=0.2, rot_dims=10, window=23), dc.moe(experts=9, top=2, ff=20, count=3, keep=1)),
-              (dc.latent(heads=5, dim=6, rot_dim=10, vdim=14, kv_rank=22, scale=0.3), dc.moe(experts=10, top=5, ff=12, count=5, keep=3)),
+              (dc.talk(heads=6, kv_heads=3, dim=20, vdim=14, scale=0.2, rot_dims=10, window=23),
+               dc.moe(experts=9, top=2, ff=20, count=3, keep=1)),
+              (dc.latent(heads=5, dim=6, rot_dim=10, vdim=14, kv_rank=22, scale=0.3),
+               dc.moe(experts=10, top=5, ff=12, count=5, keep=3)),
               (dc.talk(heads=5, kv_heads=5, dim=6, vdim=6, scale=0.5, rot_dims=2, scaling=(), window=64), dc.dense(12))]
     m = dc.Model(tmp_path, dc.config(layers, width=52, vocab=300, eps=1e-3, loop=(1, 3, 2)), seed=17)
     toks = dc.tokens(90, 300, seed=18)
@@ -438,7 +440,8 @@ def test_matrix_core_sizes(tmp_path, device):
     latent row of 160), in both dtypes; a prompt portion over several tiles and windows, then single tokens."""
     layers = [(dc.diff(heads=6, kv_heads=2, dim=32, vdim=64, scale=0.15, window=70), dc.moe(experts=12, top=3, ff=64, count=3, keep=2)),
               (dc.talk(heads=6, kv_heads=3, dim=64, vdim=64, scale=0.12, rot_dims=48, base=1e5, window=45), dc.dense(256)),
-              (dc.latent(heads=3, dim=32, rot_dim=32, vdim=48, kv_rank=128, scale=0.1, base=1e4), dc.moe(experts=8, top=3, ff=128, count=4, keep=2)),
+              (dc.latent(heads=3, dim=32, rot_dim=32, vdim=48, kv_rank=128, scale=0.1, base=1e4),
+               dc.moe(experts=8, top=3, ff=128, count=4, keep=2)),
               (dc.diff(heads=2, kv_heads=1, dim=64, vdim=128, scale=0.1, window=33), None),
               (dc.talk(heads=4, kv_heads=4, dim=64, vdim=64, scale=0.1, rot_dims=32, base=1e4, scaling=(), window=100), None)]
     m = dc.Model(tmp_path, dc.config(layers, width=128, vocab=256), seed=19)
