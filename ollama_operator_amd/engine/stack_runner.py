@@ -7,8 +7,10 @@ graphs, the sampler and the scheduler interface are the base class's. What diffe
 (`forward`: the stack executor, csrc/stack) and what a sequence owns:
 
 * every layer RUN (a repeated layer counts once per pass) has its own cache: attention runs share the
-  sequence's block table and own a K and a V pool [blocks][kv_heads][block][dim | vdim]; retention runs own
-  a float32 state [slots][heads][dim][vdim], indexed by the sequence's block-table row (its slot);
+  sequence's block table and own a K and a V pool [blocks][kv_heads][block][dim | vdim] (with several maps per
+  head a K row holds them side by side; with scores mixed across the heads the K pool has one head whose row
+  holds every key/value head's key); retention runs own a float32 state [slots][heads][dim][vdim], indexed by
+  the sequence's block-table row (its slot);
 * a slot's states are cleared when a sequence takes it, and a sequence with state keeps a cached prefix
   only whole (a state cannot be cut back), never a shorter one;
 * the residual stream is float32; matrices and the K/V pools are bfloat16 (`dtype="bfloat16"`) or
@@ -255,10 +257,12 @@ class StackRunner(Runner):
         lat = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_LATENT]
         mam = [s.mixer for s in cfg.layers if s.mixer.kind == MIX_MAMBA2]
         talk = [s.mixer for s in cfg.layers if s.mixer.talk]  # every query head against every key/value head's values
+        fold = [s.mixer for s in cfg.layers if s.mixer.score_talk]  # queries folded through the score-mixing matrix
+        maps = [s.mixer for s in cfg.layers if s.mixer.maps > 1]    # the maps' outputs before they are combined
         self.cbuf = torch.zeros(max_batch, (max([m.heads * m.cache_dim for m in lat] + [m.conv_channels for m in mam] +
                                                 [m.heads * m.kv_heads * m.vdim for m in talk] +
-                                                [max(m.heads * m.kv_heads * m.dim * m.score_talk, m.heads * m.vdim * m.maps * (m.maps > 1))
-                                                 for m in (s.mixer for s in cfg.layers)], default=1) + 3) // 4 * 4, **f32)
+                                                [m.heads * m.kv_heads * m.dim for m in fold] +
+                                                [m.heads * m.maps * m.vdim for m in maps], default=1) + 3) // 4 * 4, **f32)
         sandwich = cfg.block == BLOCK_SANDWICH
         self.hn = torch.zeros(max_batch if sandwich else 1, E, **f32)      # normed rows before the input convolution
         self.ybuf2 = torch.zeros(max_batch if sandwich else 1, E, **f32)   # the second mixer's projected output
