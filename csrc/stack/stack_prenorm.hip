@@ -206,14 +206,20 @@ __device__ __forceinline__ void route_sigmoid_wave(const MoeParams& P, const flo
   float ch = sc;
   if (P.group_count > 1) {
     const int per = P.X / P.group_count, mine = has ? lane / per : -1;
-    float gs = -INFINITY;  // this lane's group's rank
-    for (int gi = 0; gi < P.group_count; ++gi) {
-      const bool in = mine == gi;
-      const float m1 = wave_max(in ? sc : -INFINITY);
-      const int w1 = max(0, __ffsll((unsigned long long)__ballot(in && sc == m1)) - 1);
-      const float m2 = wave_max(in && lane != w1 ? sc : -INFINITY);
-      if (in) gs = m1 + (m2 == -INFINITY ? 0.f : m2);
+    // this lane's group's rank: every lane walks its own group's scores (the groups are neighbours, so one lane
+    // exchange per member) and keeps the two largest
+    const int base = has ? mine * per : lane;
+    float m1 = -INFINITY, m2 = -INFINITY;
+    for (int i = 0; i < per; ++i) {
+      const float v = __shfl(sc, has ? base + i : lane, 64);
+      if (v > m1) {
+        m2 = m1;
+        m1 = v;
+      } else if (v > m2) {
+        m2 = v;
+      }
     }
+    float gs = has ? m1 + (m2 == -INFINITY ? 0.f : m2) : -INFINITY;
     bool kept = false;
     for (int q = 0; q < P.group_keep; ++q) {
       const float best = wave_max(gs);
