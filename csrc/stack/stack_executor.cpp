@@ -555,11 +555,6 @@ void StackExecutor::layer_run(int ri, int B, hipStream_t s) {
 void StackExecutor::head(int n_logits, bool use_idx, hipStream_t s) {
   if (n_logits <= 0) return;
   if (cfg.block == 3) {  // an RMS norm with a weight vector; plain logits
-    if (!use_idx && gemv_ln_supported(n_logits, cfg.E, cfg.f32)) {  // decode steps: norm + head in one launch
-      gemv_ln(ws.resid, cfg.E, final_w, nullptr, cfg.eps, head_w, n_logits, cfg.V, in.logits, in.ld_logits, ws.lrows, nullptr, nullptr,
-              cfg.f32, s);
-      return;
-    }
     rms_norm_cast(ws.resid, use_idx ? in.logit_idx : nullptr, n_logits, cfg.E, final_w, cfg.eps, ws.lrows, cfg.f32, s);
     GemmParams g{ws.lrows, cfg.E, head_w, n_logits, cfg.V, cfg.E, in.logits, in.ld_logits, EPI_STORE, 0.f, nullptr, 0.f, cfg.f32};
     gemm(g, s);
